@@ -1,0 +1,337 @@
+"""Pins for the CPU oracle (oracle/cachegen_oracle.c).
+
+The reference holds no golden vectors for the codec (its tests assert shapes
+only), so every oracle function is pinned by checks that do not reuse its
+formula: hand-derived known answers, closed forms evaluated with a library
+(torch CPU float32 ops, numpy casts and bincount), the prefix-code closed form
+of arithmetic coding with dyadic tables, exact rational interval containment,
+and an independent bit-serial coder on Python integers (tests/pycoder.py).
+"""
+import random
+from fractions import Fraction
+
+import numpy as np
+import pytest
+import torch
+
+import pycoder
+
+
+# --------------------------------------------------------------------------- #
+# 16-bit float conversions
+# --------------------------------------------------------------------------- #
+def test_half_to_float_all_patterns(oracle):
+    L = oracle.lib()
+    bits = np.arange(65536, dtype=np.uint16)
+    want = bits.view(np.float16).astype(np.float32)
+    got = np.array([L.cgo_half_to_float(int(b)) for b in bits], dtype=np.float32)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+
+
+def test_float_to_half_rounding(oracle):
+    L = oracle.lib()
+    rng = np.random.default_rng(7)
+    cases = [0.0, -0.0, 65504.0, 65519.99, 65520.0, 1e9, -1e9, 2.0 ** -24, 2.0 ** -25,
+             2.0 ** -25 * 1.0000001, 2.0 ** -14, 2.0 ** -14 - 2.0 ** -26, 7 / 15, 1 / 3]
+    halves = np.arange(0, 0x7C00, dtype=np.uint16).view(np.float16).astype(np.float64)
+    mids = ((halves[:-1] + halves[1:]) / 2)[::37]            # exact ties
+    vals = np.concatenate([np.array(cases), mids, -mids,
+                           rng.standard_normal(4000) * 10.0 ** rng.integers(-8, 5, 4000)])
+    vals = vals.astype(np.float32)
+    want = vals.astype(np.float16).view(np.uint16)
+    got = np.array([L.cgo_float_to_half(float(v)) for v in vals], dtype=np.uint16)
+    assert np.array_equal(got, want)
+
+
+def test_bf16_conversions(oracle):
+    L = oracle.lib()
+    rng = np.random.default_rng(8)
+    vals = np.concatenate([rng.standard_normal(3000) * 10.0 ** rng.integers(-20, 20, 3000),
+                           [0.0, 1.0, 1.00390625, 1.01171875, 3.3895314e38]]).astype(np.float32)
+    t = torch.from_numpy(vals)
+    want = t.to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    got = np.array([L.cgo_float_to_bf16(float(v)) for v in vals], dtype=np.uint16)
+    assert np.array_equal(got, want)
+    back = np.array([L.cgo_bf16_to_float(int(b)) for b in want], dtype=np.float32)
+    assert np.array_equal(back, t.to(torch.bfloat16).float().numpy())
+
+
+# --------------------------------------------------------------------------- #
+# quantize / dequantize
+# --------------------------------------------------------------------------- #
+def test_quantize_known_answer(oracle):
+    # bins 32 -> MAX 15; max |x| = 1 -> factor 15; 0.5*15+15 = 22.5 rounds to even 22
+    x = np.array([[[1.0, -1.0, 0.5, 0.0]]], dtype=np.float16)
+    sym, mx = oracle.quantize(x.view(np.uint16), [32.0])
+    assert sym.tolist() == [[[30, 0, 22, 15]]]
+    assert mx.view(np.float16).tolist() == [[1.0]]
+    # bins 16 -> MAX 7: 0.5*7+7 = 10.5 -> 10 ; bins 12 -> MAX 5: 0.5*5+5 = 7.5 -> 8
+    sym, _ = oracle.quantize(np.repeat(x, 2, axis=0).view(np.uint16), [16.0, 12.0])
+    assert sym.tolist() == [[[14, 0, 10, 7]], [[10, 0, 8, 5]]]
+
+
+def test_quantize_zero_row_gives_zero_symbols(oracle):
+    x = np.zeros((1, 2, 8), dtype=np.float16)
+    x[0, 1, 3] = 2.0
+    sym, mx = oracle.quantize(x.view(np.uint16), [32.0])
+    assert sym[0, 0].tolist() == [0] * 8          # 0 * inf = nan -> int8 0
+    assert sym[0, 1].tolist() == [15, 15, 15, 30, 15, 15, 15, 15]
+    assert mx.view(np.float16).tolist() == [[0.0, 2.0]]
+
+
+def _torch_quant(x, bins):
+    """Closed form with torch CPU ops: float32 divide, multiply, add, round half even."""
+    maxq = (bins // 2 - 1)[:, None, None]
+    max1 = torch.amax(torch.abs(x), dim=-1, keepdim=True)
+    factor = maxq / max1
+    return torch.round(x * factor + maxq).to(torch.int8), max1
+
+
+@pytest.mark.parametrize("dtype,dt", [(torch.float16, 0), (torch.bfloat16, 1)])
+def test_quantize_matches_torch_float32_ops(oracle, dtype, dt):
+    g = torch.Generator().manual_seed(11)
+    x = (torch.randn(5, 37, 96, generator=g) * torch.exp(torch.randn(5, 1, 96, generator=g))).to(dtype)
+    x[2, 5] *= 1e-4                                 # a tiny row
+    x[3, 7, 11] = 300.0                             # an outlier
+    bins = torch.tensor([32.0, 32.0, 16.0, 12.0, 8.0])
+    want_sym, want_max = _torch_quant(x, bins)
+    sym, mx = oracle.quantize(x.view(torch.int16).numpy().view(np.uint16), bins.numpy(), dt)
+    assert np.array_equal(sym, want_sym.numpy().view(np.uint8))
+    assert np.array_equal(mx, want_max[..., 0].view(torch.int16).numpy().view(np.uint16))
+    assert int(sym.max()) <= 30 and sym[2:3].max() <= 14 and sym[3:4].max() <= 10
+
+
+def test_dequantize_known_answer(oracle):
+    # s=22, C=15, max=1 -> fp32 7/15 -> nearest fp16
+    out = oracle.dequantize(np.array([[[22, 0, 30, 15]]], dtype=np.uint8), [32.0],
+                            np.array([[1.0]], dtype=np.float16).view(np.uint16))
+    want = np.array([np.float32(7) / np.float32(15), -1.0, 1.0, 0.0], dtype=np.float32).astype(np.float16)
+    assert np.array_equal(out[0, 0].view(np.float16), want)
+
+
+@pytest.mark.parametrize("max_dtype,max_dt", [(torch.float16, 0), (torch.bfloat16, 1)])
+@pytest.mark.parametrize("out_dtype,out_dt", [(torch.float16, 0), (torch.bfloat16, 1)])
+def test_dequantize_matches_torch_float32_ops(oracle, max_dtype, max_dt, out_dtype, out_dt):
+    g = torch.Generator().manual_seed(12)
+    bins = torch.tensor([32.0, 16.0, 12.0])
+    sym = torch.stack([torch.randint(0, int(b) - 1, (23, 40), generator=g) for b in bins]).to(torch.uint8)
+    maxima = (torch.rand(3, 23, 1, generator=g) * 20 + 1e-3).to(max_dtype)
+    maxima[1, 4] = 6e-6                              # result lands in the fp16 subnormals
+    c = (bins // 2 - 1)[:, None, None]
+    want = (((sym.float() - c) / c) * maxima).to(out_dtype)
+    got = oracle.dequantize(sym.numpy(), bins.numpy(),
+                            maxima[..., 0].view(torch.int16).numpy().view(np.uint16), max_dt, out_dt)
+    assert np.array_equal(got, want.view(torch.int16).numpy().view(np.uint16))
+
+
+# --------------------------------------------------------------------------- #
+# CDF
+# --------------------------------------------------------------------------- #
+def test_cdf_known_answer(oracle):
+    # max_bins 32, T 4, symbols [0,0,1,30]: cum = [0,2,3,...,3,4,4];
+    # cdf[i] = floor(65503*cum[i]/4) + i
+    sym = np.array([0, 0, 1, 30], dtype=np.uint8).reshape(1, 4, 1)
+    cdf = oracle.calculate_cdf(sym, 32)[0, 0].tolist()
+    want = [0, 32751 + 1] + [49127 + i for i in range(2, 31)] + [65503 + 31, 65503 + 32]
+    assert cdf == want and cdf[32] == 65535 and cdf[31] == 65534
+
+
+@pytest.mark.parametrize("max_bins,nt", [(32, 256), (32, 1500), (16, 7), (63, 900), (12, 65535)])
+def test_cdf_matches_integer_bincount(oracle, max_bins, nt):
+    rng = np.random.default_rng(max_bins * 1000 + nt)
+    nl, nc = 2, 9
+    p = rng.dirichlet(np.ones(max_bins - 1) * 0.3, size=(nl, nc))
+    sym = np.empty((nl, nt, nc), dtype=np.uint8)
+    for l in range(nl):
+        for c in range(nc):
+            sym[l, :, c] = rng.choice(max_bins - 1, size=nt, p=p[l, c])
+    cdf = oracle.calculate_cdf(sym, max_bins)
+    for l in range(nl):
+        for c in range(nc):
+            counts = np.bincount(sym[l, :, c], minlength=max_bins)[:max_bins]
+            cum = [0] + [int(v) for v in np.cumsum(counts)]
+            want = [((0xFFFF - max_bins) * cum[i]) // nt + i for i in range(max_bins + 1)]
+            assert cdf[l, c].tolist() == want
+            assert all(b > a for a, b in zip(want, want[1:]))        # strictly increasing
+            assert want[0] == 0 and want[-1] == 65535
+
+
+def test_cdf_honours_strides(oracle):
+    rng = np.random.default_rng(3)
+    big = rng.integers(0, 31, size=(3, 40, 10), dtype=np.uint8)
+    view = big[:, 8:29, :]
+    assert np.array_equal(oracle.calculate_cdf(view, 32), oracle.calculate_cdf(view.copy(), 32))
+
+
+# --------------------------------------------------------------------------- #
+# arithmetic coder
+# --------------------------------------------------------------------------- #
+def test_coder_hand_known_answers(oracle):
+    cdf = [0, 32768, 65535]
+    # symbol 0 halves the range to the lower half: emits 0; the tail emits 0,1 -> 001 00000
+    assert oracle.encode_stream(cdf, [0]) == (bytes([0x20]), 1)
+    # symbol 1 (= Lp-2, upper bound 0x10000): emits 1 then 0,1 -> 101 00000
+    assert oracle.encode_stream(cdf, [1]) == (bytes([0xA0]), 1)
+    assert oracle.decode_stream(cdf, bytes([0x20]), 1).tolist() == [0]
+    assert oracle.decode_stream(cdf, bytes([0xA0]), 1).tolist() == [1]
+    # middle-half symbol [1/4, 3/4): one pending bit; then symbol 0 ([0, 1/4)) resolves it:
+    # "01" + "0", tail "01" -> 01001 000
+    cdf3 = [0, 16384, 49152, 65535]
+    assert oracle.encode_stream(cdf3, [1, 0]) == (bytes([0x48]), 1)
+    # [1/4,3/4) then its upper quarter [5/8,3/4) -> binary 0.101 ; tail 01 -> 10101 000
+    assert oracle.encode_stream(cdf3, [1, 2]) == (bytes([0xA8]), 1)
+    assert oracle.decode_stream(cdf3, bytes([0x48]), 2).tolist() == [1, 0]
+    assert oracle.decode_stream(cdf3, bytes([0xA8]), 2).tolist() == [1, 2]
+    # empty stream: only the tail "01"
+    assert oracle.encode_stream(cdf, []) == (bytes([0x40]), 1)
+
+
+def test_coder_long_pending_run(oracle):
+    # [1/4,3/4) forty times keeps the range straddling the midpoint: 40 pending bits that
+    # the tail resolves as 0 followed by 41 ones (crosses a 32-bit register flush).
+    cdf3 = [0, 16384, 49152, 65535]
+    data, n = oracle.encode_stream(cdf3, [1] * 40)
+    bits = "0" + "1" * 41
+    bits += "0" * (-len(bits) % 8)
+    assert data == int(bits, 2).to_bytes(len(bits) // 8, "big") and n == len(bits) // 8
+    assert oracle.decode_stream(cdf3, data, 40).tolist() == [1] * 40
+    # ... and when a lower-quarter symbol resolves them: 0, 40 ones, 0, then tail 01
+    data, _ = oracle.encode_stream(cdf3, [1] * 40 + [0])
+    bits = "0" + "1" * 40 + "0" + "01"
+    bits += "0" * (-len(bits) % 8)
+    assert data == int(bits, 2).to_bytes(len(bits) // 8, "big")
+
+
+def _random_prefix_code(rng, nleaves, max_depth=14):
+    """Leaves of a random full binary tree, left to right, as (codeword, depth)."""
+    leaves = [(0, 0)]
+    while len(leaves) < nleaves:
+        i = rng.randrange(len(leaves))
+        code, d = leaves[i]
+        if d >= max_depth:
+            continue
+        leaves[i:i + 1] = [(code << 1, d + 1), ((code << 1) | 1, d + 1)]
+    return leaves
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_coder_equals_prefix_code_for_dyadic_tables(oracle, seed):
+    """With a table whose intervals are nodes of a binary tree the coder is exact and
+    emits each symbol's codeword; the tail adds "01" and zero padding."""
+    rng = random.Random(seed)
+    nsym = rng.choice([2, 3, 5, 8, 15, 31])
+    leaves = _random_prefix_code(rng, nsym)
+    cdf = [code << (16 - d) for code, d in leaves] + [65535]
+    weights = [2.0 ** -d for _, d in leaves]
+    for n in (1, 7, 64, 256):
+        syms = rng.choices(range(nsym), weights=weights, k=n)
+        bits = "".join(format(leaves[s][0], "0%db" % leaves[s][1]) if leaves[s][1] else "" for s in syms)
+        bits += "01"
+        bits += "0" * (-len(bits) % 8)
+        want = int(bits, 2).to_bytes(len(bits) // 8, "big")
+        got, length = oracle.encode_stream(cdf, syms, cap=4096)
+        assert got == want and length == len(want)
+        assert oracle.decode_stream(cdf, want, n).tolist() == syms
+
+
+@pytest.mark.parametrize("seed", range(5))
+def test_coder_output_lies_in_exact_interval(oracle, seed):
+    """Tables with power-of-two widths at arbitrary positions keep the integer coder exact
+    (no truncation), so the emitted number and every continuation of it must lie inside the
+    rational interval of the message.  Exercises the pending-bit path."""
+    rng = random.Random(100 + seed)
+    # widths 2^-k summing to 1, shuffled so that intervals are not tree nodes
+    widths = [1 << 14] * 2 + [1 << 13] * 2 + [1 << 12] * 4
+    rng.shuffle(widths)
+    cdf = [0]
+    for w in widths:
+        cdf.append(cdf[-1] + w)
+    assert cdf[-1] == 65536
+    cdf[-1] = 65535
+    edges = cdf[:-1] + [65536]
+    for n in (3, 9, 12):
+        syms = [rng.randrange(len(widths)) for _ in range(n)]
+        lo, width = Fraction(0), Fraction(1)
+        for s in syms:
+            lo += width * Fraction(edges[s], 65536)
+            width *= Fraction(edges[s + 1] - edges[s], 65536)
+        data, _ = oracle.encode_stream(cdf, syms)
+        x = Fraction(int.from_bytes(data, "big"), 1 << (8 * len(data)))
+        assert lo <= x and x + Fraction(1, 1 << (8 * len(data))) <= lo + width
+        assert oracle.decode_stream(cdf, data, n).tolist() == syms
+
+
+def _random_table(rng, lp):
+    cuts = sorted(rng.sample(range(1, 65535), lp - 2))
+    return [0] + cuts + [65535]
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_coder_matches_independent_python_coder(oracle, seed):
+    rng = random.Random(200 + seed)
+    lp = rng.choice([3, 4, 13, 17, 33, 33, 48, 65])
+    cdf = _random_table(rng, lp)
+    widths = [b - a for a, b in zip(cdf[:-2], cdf[1:-1])] + [65536 - cdf[-2]]
+    for n in (1, 2, 31, 256):
+        syms = rng.choices(range(lp - 1), weights=widths, k=n)
+        if seed % 2:
+            syms = [rng.randrange(lp - 1) for _ in range(n)]       # improbable symbols too
+        want, _ = pycoder.encode(cdf, syms)
+        got, length = oracle.encode_stream(cdf, syms, cap=8192)
+        assert got == want and length == len(want)
+        assert pycoder.decode(cdf, want, n) == syms
+        assert oracle.decode_stream(cdf, want, n).tolist() == syms
+
+
+def test_coder_on_calculated_tables_round_trip_and_size(oracle):
+    """Tables from calculate_cdf over 1500 tokens, 256-token streams: round trip, and the
+    length is the empirical cross entropy plus at most a few bytes."""
+    rng = np.random.default_rng(5)
+    nl, nt, nc = 2, 1500, 24
+    p = rng.dirichlet(np.ones(31) * 0.4, size=(nl, nc))
+    sym = np.empty((nl, nt, nc), dtype=np.uint8)
+    for l in range(nl):
+        for c in range(nc):
+            sym[l, :, c] = rng.choice(31, size=nt, p=p[l, c])
+    cdf = oracle.calculate_cdf(sym, 32)
+    part = sym[:, 256:512, :]
+    padded, lengths = oracle.encode_fast_new(cdf, part)
+    assert lengths.min() >= 1 and lengths.max() <= 256
+    for l in range(nl):
+        for c in range(nc):
+            row = cdf[l, c].astype(np.int64)
+            w = np.diff(np.append(row[:-1], 65536))
+            bits = -np.log2(w[part[l, :, c]] / 65536.0).sum()
+            assert bits / 8 <= lengths[l, c] <= bits / 8 + 2
+            want, _ = pycoder.encode(row.tolist(), part[l, :, c].tolist())
+            assert padded[l, c, :lengths[l, c]].tobytes() == want
+    data = oracle.collect_bytes(padded, lengths)
+    assert data.tobytes() == b"".join(padded[l, c, :lengths[l, c]].tobytes()
+                                      for l in range(nl) for c in range(nc))
+    prefix = lengths.astype(np.int64).ravel().cumsum().reshape(lengths.shape)
+    assert np.array_equal(oracle.decode_fast_prefsum(cdf, data, prefix, 256), part)
+    assert np.array_equal(oracle.decode_fast_new(cdf, padded, lengths, 256), part)
+
+
+def test_encode_leaves_bytes_past_length_untouched(oracle):
+    cdf = np.array([[[0, 32768, 65535]]], dtype=np.uint16)
+    sym = np.zeros((1, 3, 1), dtype=np.uint8)
+    out = np.full((1, 1, 256), 0xEE, dtype=np.uint8)
+    out, lengths = oracle.encode_fast_new(cdf, sym, out)
+    assert lengths[0, 0] == 1 and out[0, 0, 0] == 0x08 and (out[0, 0, 1:] == 0xEE).all()
+
+
+def test_end_to_end_functions_round_trip(oracle):
+    from cachegen_amd.kvgen import make_kv
+    kv = make_kv(2, 300, 2, 16, seed=9)
+    bits = kv.reshape(2, 2, 300, 32).view(torch.int16).numpy().view(np.uint16)
+    enc = oracle.encode_function(bits, [32.0, 16.0], [32.0, 16.0])
+    assert [c[2] for c in enc["data_chunks"]] == [256, 44]
+    sym, out = oracle.decode_function(enc, [32.0, 16.0], [32.0, 16.0])
+    assert np.array_equal(sym, enc["symbols"])
+    x = kv.reshape(2, 2, 300, 32).float()
+    y = torch.from_numpy(out.view(np.int16)).view(torch.float16).float()
+    step = x.abs().amax(dim=-1, keepdim=True) / torch.tensor([15.0, 7.0])[:, None, None, None]
+    assert bool(((x - y).abs() <= step * 0.5 + 1e-3).all())

@@ -1,0 +1,1214 @@
+// CacheGen KV codec for MI355X (gfx950): hand-written HIP kernels behind a C ABI.
+//
+// The codec is HBM/ALU-bound integer work with no dense contraction, so there is
+// no MFMA here.  The mapping everywhere is one lane = one (row, channel) stream
+// and one wavefront = 64 adjacent channels of one row, which keeps every symbol
+// and KV access of a wave on one contiguous segment; per-wave tables live in LDS
+// as [entry][lane] 32-bit words so that lanes never collide on a bank.
+//
+// Paths in the comments are relative to LMCache/ in the reference tree:
+//   enc_new.cu = third_party/torchac_cuda/torchac_kernel_enc_new.cu
+//   dec_new.cu = third_party/torchac_cuda/torchac_kernel_dec_new.cu
+//   cal_cdf.cu = third_party/torchac_cuda/cal_cdf.cu
+//   encoder.py = lmcache/storage_backend/serde/cachegen_encoder.py
+//   decoder.py = lmcache/storage_backend/serde/cachegen_decoder.py
+#include <hip/hip_runtime.h>
+
+#include <climits>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "cachegen_hip.h"
+
+// The float32 steps of quantisation and dequantisation are rounded one by one, as eager
+// tensor code rounds them: no fused multiply-add anywhere in this file.
+#pragma clang fp contract(off)
+
+namespace {
+
+// ------------------------------------------------------------------------------------
+// host-side helpers
+// ------------------------------------------------------------------------------------
+thread_local char g_error[512] = "";
+
+int fail(int code, const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int check_launch(const char *what)
+{
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(CG_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+    return CG_OK;
+}
+
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+inline bool aligned_to(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+constexpr int kSub = CG_MAX_TOKENS_PER_STREAM;   // tokens per stream (cachegen_basics.py:8)
+constexpr int kStreamCap = 256;                  // bytes kept per stream in the fused path
+
+// Token geometry shared by the stream kernels: chunk k covers tokens
+// [k*S, min((k+1)*S, T)), and is cut every 256 tokens (encoder.py:279-292).
+struct TokenGeom {
+    int64_t T;        // tokens in the tensor
+    int64_t S;        // tokens per chunk (one table per chunk)
+    int32_t nsc;      // sub-chunks in a full chunk = ceil(S / 256)
+};
+
+__host__ __device__ inline void sub_range(const TokenGeom &g, int64_t sub, int64_t &chunk,
+                                          int64_t &t0, int &n)
+{
+    chunk = sub / g.nsc;
+    const int64_t j = sub - chunk * g.nsc;
+    t0 = chunk * g.S + j * kSub;
+    int64_t tend = (chunk + 1) * g.S;
+    if (tend > g.T) tend = g.T;
+    const int64_t left = tend - t0;
+    n = left < kSub ? (int)left : kSub;
+}
+
+// ------------------------------------------------------------------------------------
+// device helpers
+// ------------------------------------------------------------------------------------
+__device__ __forceinline__ float f16_bits_to_float(uint32_t h)
+{
+    _Float16 v;
+    uint16_t b = (uint16_t)h;
+    __builtin_memcpy(&v, &b, 2);
+    return (float)v;
+}
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t h) { return __uint_as_float(h << 16); }
+
+template <int DT>
+__device__ __forceinline__ float load16f(uint32_t bits)
+{
+    return DT == CG_DT_BF16 ? bf16_bits_to_float(bits) : f16_bits_to_float(bits);
+}
+
+__device__ __forceinline__ uint32_t float_to_f16_bits(float f)
+{
+    _Float16 v = (_Float16)f;      // v_cvt_f16_f32, round to nearest even
+    uint16_t b;
+    __builtin_memcpy(&b, &v, 2);
+    return b;
+}
+__device__ __forceinline__ uint32_t float_to_bf16_bits(float f)
+{
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (u >> 16) | 0x40u;
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+template <int DT>
+__device__ __forceinline__ uint32_t store16f(float f)
+{
+    return DT == CG_DT_BF16 ? float_to_bf16_bits(f) : float_to_f16_bits(f);
+}
+
+// floor(span * c / 2^16) for span = r + 1 (rh = r >> 16, rl = r & 0xffff) and a table
+// value c <= 0xffff, on the full-rate 24-bit multiplier: span*c = rh*c*2^16 + (rl+1)*c.
+// This is `(span * c) >> precision` of enc_new.cu:272-273 / dec_new.cu:280-281.
+__device__ __forceinline__ uint32_t scale16(uint32_t rh, uint32_t rl, uint32_t c)
+{
+    const uint32_t lowpart = __umul24(rl, c) + c;
+    return __umul24(rh, c) + (lowpart >> 16);
+}
+
+// ------------------------------------------------------------------------------------
+// Quantization (encoder.py:42-59): one wavefront per (row of 2L, token).
+// Each lane holds up to 8 units of 8 channels (one 128-bit load each) in registers, the
+// row maximum of |x| is an integer maximum of the sign-stripped 16-bit patterns (two per
+// packed op), and the float32 operations are the reference's, each rounded separately:
+//   factor = MAX / max ; sym = rint(x * factor + MAX)
+// ------------------------------------------------------------------------------------
+constexpr int kMaxUnits = 8;
+
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b)
+{
+    typedef unsigned short us2 __attribute__((ext_vector_type(2)));
+    us2 x, y;
+    __builtin_memcpy(&x, &a, 4);
+    __builtin_memcpy(&y, &b, 4);
+    us2 z = __builtin_elementwise_max(x, y);
+    uint32_t r;
+    __builtin_memcpy(&r, &z, 4);
+    return r;
+}
+
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v)
+{
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) {
+        uint32_t other = (uint32_t)__shfl_xor((int)v, o, 64);
+        v = other > v ? other : v;
+    }
+    return v;
+}
+
+template <int DT>
+__device__ __forceinline__ uint32_t quant_one(uint32_t bits, float factor, float maxq)
+{
+    const float v = load16f<DT>(bits);
+    const float p = __fmul_rn(v, factor);
+    const float s = __fadd_rn(p, maxq);
+    float r = __builtin_rintf(s);
+    r = (r != r) ? 0.0f : r;          // 0 * inf of an all-zero row: int8 cast of NaN is 0
+    return (uint32_t)(int)r & 0xFFu;
+}
+
+template <int DT, bool HEADS_CONTIGUOUS>
+__global__ __launch_bounds__(256) void quantize_kv_kernel(
+    const uint16_t *__restrict__ kv, int64_t L, int64_t T, int D, int64_t sl, int64_t skv,
+    int64_t st, int64_t sh, const float *__restrict__ key_bins,
+    const float *__restrict__ value_bins, uint8_t *__restrict__ sym,
+    uint16_t *__restrict__ maxima, int nunits, int64_t nrows)
+{
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + wave;
+    if (row >= nrows) return;
+    const int64_t layer2 = row / T, t = row - layer2 * T;
+    const int64_t kvi = layer2 / L, l = layer2 - kvi * L;
+    const uint16_t *base = kv + l * sl + kvi * skv + t * st;
+    const float bins = (kvi ? value_bins : key_bins)[l];
+    const float maxq = floorf(bins * 0.5f) - 1.0f;
+
+    uint4 regs[kMaxUnits];
+    uint32_t m = 0;
+#pragma unroll
+    for (int i = 0; i < kMaxUnits; ++i) {
+        const int u = lane + 64 * i;
+        if (u < nunits) {
+            const int e = u * 8;
+            int64_t off;
+            if (HEADS_CONTIGUOUS) off = e;
+            else { const int h = e / D; off = (int64_t)h * sh + (e - h * D); }
+            regs[i] = *reinterpret_cast<const uint4 *>(base + off);
+            m = pk_max_u16(m, regs[i].x & 0x7FFF7FFFu);
+            m = pk_max_u16(m, regs[i].y & 0x7FFF7FFFu);
+            m = pk_max_u16(m, regs[i].z & 0x7FFF7FFFu);
+            m = pk_max_u16(m, regs[i].w & 0x7FFF7FFFu);
+        }
+    }
+    m = (m & 0xFFFFu) > (m >> 16) ? (m & 0xFFFFu) : (m >> 16);
+    m = wave_max_u32(m);
+    if (lane == 0) maxima[row] = (uint16_t)m;
+    const float factor = __fdiv_rn(maxq, load16f<DT>(m));
+
+    uint8_t *out = sym + row * ((int64_t)nunits * 8);
+#pragma unroll
+    for (int i = 0; i < kMaxUnits; ++i) {
+        const int u = lane + 64 * i;
+        if (u < nunits) {
+            const uint32_t w[4] = {regs[i].x, regs[i].y, regs[i].z, regs[i].w};
+            uint32_t q[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                q[j] = quant_one<DT>(w[2 * j] & 0xFFFFu, factor, maxq) |
+                       (quant_one<DT>(w[2 * j] >> 16, factor, maxq) << 8) |
+                       (quant_one<DT>(w[2 * j + 1] & 0xFFFFu, factor, maxq) << 16) |
+                       (quant_one<DT>(w[2 * j + 1] >> 16, factor, maxq) << 24);
+            }
+            *reinterpret_cast<uint2 *>(out + (int64_t)u * 8) = make_uint2(q[0], q[1]);
+        }
+    }
+}
+
+// Any shape / alignment: one wavefront per row, two passes over global memory.
+template <int DT>
+__global__ __launch_bounds__(256) void quantize_kv_generic_kernel(
+    const uint16_t *__restrict__ kv, int64_t L, int64_t T, int D, int C, int64_t sl, int64_t skv,
+    int64_t st, int64_t sh, const float *__restrict__ key_bins,
+    const float *__restrict__ value_bins, uint8_t *__restrict__ sym,
+    uint16_t *__restrict__ maxima, int64_t nrows)
+{
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + wave;
+    if (row >= nrows) return;
+    const int64_t layer2 = row / T, t = row - layer2 * T;
+    const int64_t kvi = layer2 / L, l = layer2 - kvi * L;
+    const uint16_t *base = kv + l * sl + kvi * skv + t * st;
+    const float bins = (kvi ? value_bins : key_bins)[l];
+    const float maxq = floorf(bins * 0.5f) - 1.0f;
+    uint32_t m = 0;
+    for (int c = lane; c < C; c += 64) {
+        const int h = c / D;
+        const uint32_t b = base[(int64_t)h * sh + (c - h * D)] & 0x7FFFu;
+        m = b > m ? b : m;
+    }
+    m = wave_max_u32(m);
+    if (lane == 0) maxima[row] = (uint16_t)m;
+    const float factor = __fdiv_rn(maxq, load16f<DT>(m));
+    uint8_t *out = sym + row * (int64_t)C;
+    for (int c = lane; c < C; c += 64) {
+        const int h = c / D;
+        out[c] = (uint8_t)quant_one<DT>(base[(int64_t)h * sh + (c - h * D)], factor, maxq);
+    }
+}
+
+// ------------------------------------------------------------------------------------
+// Tables (cal_cdf.cu:17-59): one lane per (chunk, row, channel) walks the chunk's tokens
+// and counts into its own LDS column hist[bin][lane] (no atomics, no bank conflicts);
+// the running sum and the normalisation
+//   cdf[i] = (uint16)((0xFFFF - max_bins) * cum[i] / cum[max_bins]) + i
+// are done per lane in 16-bit wrap-around arithmetic like the reference's uint16
+// counters, and the wave writes its 64 tables back transposed so stores coalesce.
+// ------------------------------------------------------------------------------------
+struct CdfArgs {
+    const uint8_t *sym;
+    int64_t s0, s1, s2;     // sym[row*s0 + token*s1 + channel*s2]
+    uint16_t *cdf;          // [chunk][row][channel][lp]
+    int64_t rows, nc;
+    int32_t ctiles;         // blocks per row
+    int32_t max_bins;
+    TokenGeom g;
+};
+
+__global__ __launch_bounds__(256) void calculate_cdf_kernel(CdfArgs a)
+{
+    extern __shared__ uint32_t smem[];
+    const int bs = blockDim.x, tid = threadIdx.x;
+    const int lp = a.max_bins + 1;
+    int64_t b = blockIdx.x;
+    const int ctile = (int)(b % a.ctiles);
+    b /= a.ctiles;
+    const int64_t row = b % a.rows;
+    const int64_t chunk = b / a.rows;
+    const int64_t ch = (int64_t)ctile * bs + tid;
+    const bool active = ch < a.nc;
+
+    for (int i = 0; i < lp; ++i) smem[i * bs + tid] = 0;
+
+    const int64_t t0 = chunk * a.g.S;
+    int64_t t1 = t0 + a.g.S;
+    if (t1 > a.g.T) t1 = a.g.T;
+    if (active) {
+        const uint8_t *p = a.sym + row * a.s0 + ch * a.s2;
+        int64_t t = t0;
+        for (; t + 4 <= t1; t += 4) {
+            const uint32_t v0 = p[(t + 0) * a.s1], v1 = p[(t + 1) * a.s1];
+            const uint32_t v2 = p[(t + 2) * a.s1], v3 = p[(t + 3) * a.s1];
+            if (v0 < (uint32_t)a.max_bins) smem[(v0 + 1) * bs + tid]++;
+            if (v1 < (uint32_t)a.max_bins) smem[(v1 + 1) * bs + tid]++;
+            if (v2 < (uint32_t)a.max_bins) smem[(v2 + 1) * bs + tid]++;
+            if (v3 < (uint32_t)a.max_bins) smem[(v3 + 1) * bs + tid]++;
+        }
+        for (; t < t1; ++t) {
+            const uint32_t v = p[t * a.s1];
+            if (v < (uint32_t)a.max_bins) smem[(v + 1) * bs + tid]++;
+        }
+        uint32_t running = 0;
+        for (int i = 1; i < lp; ++i) {
+            running = (running + smem[i * bs + tid]) & 0xFFFFu;
+            smem[i * bs + tid] = running;
+        }
+        const uint32_t scale = 0xFFFFu - (uint32_t)a.max_bins;
+        for (int i = 0; i < lp; ++i) {
+            const uint32_t q = running ? (scale * smem[i * bs + tid] / running) & 0xFFFFu : 0u;
+            smem[i * bs + tid] = (q + (uint32_t)i) & 0xFFFFu;
+        }
+    }
+    __syncthreads();
+    const int64_t ch0 = (int64_t)ctile * bs;
+    const int64_t nvalid = (a.nc - ch0 < bs) ? (a.nc - ch0) : bs;
+    uint16_t *out = a.cdf + ((chunk * a.rows + row) * a.nc + ch0) * lp;
+    const int total = (int)nvalid * lp;
+    for (int i = tid; i < total; i += bs) {
+        const int c = i / lp, e = i - c * lp;
+        out[i] = (uint16_t)smem[e * bs + c];
+    }
+}
+
+// ------------------------------------------------------------------------------------
+// Arithmetic coder.  Shared geometry of the encoder and decoder kernels: a block of
+// `blockDim.x` lanes covers that many adjacent channels of one (sub-chunk, row).
+// ------------------------------------------------------------------------------------
+struct StreamGrid {
+    int64_t rows, nc;
+    int32_t ctiles;
+    TokenGeom g;
+};
+
+struct StreamId {
+    int64_t sub, row, chunk, t0, ch;
+    int n;
+    bool active;
+};
+
+__device__ __forceinline__ StreamId locate(const StreamGrid &sg)
+{
+    StreamId s;
+    int64_t b = blockIdx.x;
+    const int ctile = (int)(b % sg.ctiles);
+    b /= sg.ctiles;
+    s.row = b % sg.rows;
+    s.sub = b / sg.rows;
+    sub_range(sg.g, s.sub, s.chunk, s.t0, s.n);
+    s.ch = (int64_t)ctile * blockDim.x + threadIdx.x;
+    s.active = s.ch < sg.nc;
+    return s;
+}
+
+// Load the block's tables into LDS as tab[entry * bs + lane] (32-bit words).
+__device__ __forceinline__ void stage_tables(uint32_t *tab, const uint16_t *cdf, int lp,
+                                             int64_t ch0, int64_t nc)
+{
+    const int bs = blockDim.x;
+    const int64_t nvalid = (nc - ch0 < bs) ? (nc - ch0) : bs;
+    const int total = (int)nvalid * lp;
+    for (int i = threadIdx.x; i < total; i += bs) {
+        const int c = i / lp, e = i - c * lp;
+        tab[e * bs + c] = cdf[i];
+    }
+}
+
+// ---- encoder (enc_new.cu:21-97, 253-307) -------------------------------------------
+// Bits are collected MSB-first in a 32-bit accumulator and leave as big-endian words.
+// The E1/E2 run of a symbol is emitted at once: clz(low ^ high) leading bits agree, the
+// first of them is followed by the pending complements; the E3 run is the number of
+// positions below the top where low has ones and high has zeros.
+template <bool ALIGNED>
+struct BitWriter {
+    uint8_t *dst;
+    int cap;
+    int nbytes;
+    uint32_t acc;
+    int nacc;
+
+    __device__ __forceinline__ void store_word(uint32_t word)
+    {
+        if (nbytes + 4 <= cap) {
+            if (ALIGNED) {
+                *reinterpret_cast<uint32_t *>(dst + nbytes) = __builtin_bswap32(word);
+            } else {
+                dst[nbytes + 0] = (uint8_t)(word >> 24);
+                dst[nbytes + 1] = (uint8_t)(word >> 16);
+                dst[nbytes + 2] = (uint8_t)(word >> 8);
+                dst[nbytes + 3] = (uint8_t)word;
+            }
+        } else {
+            for (int j = 0; j < 4; ++j)
+                if (nbytes + j < cap) dst[nbytes + j] = (uint8_t)(word >> (24 - 8 * j));
+        }
+        nbytes += 4;
+    }
+
+    // append the low m bits of v (v < 2^m), 1 <= m <= 32
+    __device__ __forceinline__ void put(uint32_t v, int m)
+    {
+        const int tot = nacc + m;
+        if (tot < 32) {
+            acc = (acc << m) | v;
+            nacc = tot;
+        } else {
+            const uint32_t vl = v << (32 - m);
+            store_word(__builtin_amdgcn_alignbit(acc, vl, (uint32_t)nacc));
+            nacc = tot - 32;
+            acc = v & ((1u << nacc) - 1u);
+        }
+    }
+
+    __device__ __forceinline__ void run(uint32_t bit, uint32_t count)
+    {
+        while (count > 0) {
+            const int take = count < 32u ? (int)count : 32;
+            const uint32_t ones = take == 32 ? 0xFFFFFFFFu : ((1u << take) - 1u);
+            put(bit ? ones : 0u, take);
+            count -= (uint32_t)take;
+        }
+    }
+
+    // write the partial accumulator (enc_new.cu:42-55); returns the stream length
+    __device__ __forceinline__ int finish()
+    {
+        if (nacc > 0) {
+            uint32_t r = acc << (32 - nacc);
+            for (int left = nacc; left > 0; left -= 8) {
+                if (nbytes < cap) dst[nbytes] = (uint8_t)(r >> 24);
+                nbytes++;
+                r <<= 8;
+            }
+        }
+        return nbytes;
+    }
+};
+
+struct EncodeArgs {
+    const uint16_t *cdf;    // [chunk][row][channel][lp]
+    int32_t lp;
+    const uint8_t *sym;     // sym[row*s0 + token*s1 + channel*s2]
+    int64_t s0, s1, s2;
+    uint8_t *out;           // out[sub*osub + row*o0 + channel*o1 + byte]
+    int64_t osub, o0, o1;
+    int32_t cap;
+    int32_t *lengths;       // [sub][row][channel]
+    int32_t *status;        // may be null
+    StreamGrid sg;
+};
+
+template <bool ALIGNED>
+__global__ __launch_bounds__(256) void encode_streams_kernel(EncodeArgs a)
+{
+    extern __shared__ uint32_t tab[];
+    const int bs = blockDim.x, tid = threadIdx.x;
+    const StreamId id = locate(a.sg);
+    const int lp = a.lp;
+    const int64_t ch0 = id.ch - tid;
+    stage_tables(tab, a.cdf + ((id.chunk * a.sg.rows + id.row) * a.sg.nc + ch0) * lp, lp, ch0, a.sg.nc);
+    __syncthreads();
+    if (!id.active) return;
+    // the upper bound of the last symbol is 2^16, not the stored value (enc_new.cu:270)
+    tab[(lp - 1) * bs + tid] = 0x10000u;
+
+    const uint8_t *sp = a.sym + id.row * a.s0 + id.t0 * a.s1 + id.ch * a.s2;
+    BitWriter<ALIGNED> w;
+    w.dst = a.out + id.sub * a.osub + id.row * a.o0 + id.ch * a.o1;
+    w.cap = a.cap;
+    w.nbytes = 0;
+    w.acc = 0;
+    w.nacc = 0;
+
+    uint32_t low = 0, high = 0xFFFFFFFFu, pend = 0;
+    const uint32_t top = (uint32_t)(lp - 1);
+    uint32_t s_next = id.n > 0 ? sp[0] : 0;
+    for (int i = 0; i < id.n; ++i) {
+        uint32_t s = s_next;
+        if (i + 1 < id.n) s_next = sp[(int64_t)(i + 1) * a.s1];
+        s = s < top ? s : top - 1;                      // keep table reads inside the table
+        const uint32_t r = high - low;
+        const uint32_t rh = r >> 16, rl = r & 0xFFFFu;
+        const uint32_t c_lo = tab[s * bs + tid];
+        const uint32_t c_hi = tab[(s + 1) * bs + tid];
+        const uint32_t t_lo = scale16(rh, rl, c_lo);
+        const uint32_t t_hi = c_hi == 0x10000u ? r + 1u : scale16(rh, rl, c_hi);
+        high = low + t_hi - 1u;
+        low = low + t_lo;
+
+        const int n1 = __builtin_clz(low ^ high);        // low < high always
+        if (n1 > 0) {
+            const uint32_t b = low >> 31;
+            const uint32_t rest = (low & 0x7FFFFFFFu) >> (32 - n1);
+            if (pend + (uint32_t)n1 <= 32u) {
+                const uint32_t head = ((1u << pend) - 1u) + b;   // b, then `pend` complements
+                w.put((head << (n1 - 1)) | rest, (int)pend + n1);
+            } else {
+                w.put(b, 1);
+                w.run(1u - b, pend);
+                if (n1 > 1) w.put(rest, n1 - 1);
+            }
+            pend = 0;
+        }
+        const uint32_t lo1 = low << n1;
+        const uint32_t hi1 = (high << n1) | ((1u << n1) - 1u);
+        const int k = __builtin_clz(~((lo1 & ~hi1) << 1));
+        pend += (uint32_t)k;
+        low = (lo1 << k) & 0x7FFFFFFFu;
+        high = (hi1 << k) | 0x80000000u | ((1u << k) - 1u);
+    }
+    pend += 1;
+    const uint32_t b = low < 0x40000000u ? 0u : 1u;
+    w.put(b, 1);
+    w.run(1u - b, pend);
+    const int len = w.finish();
+    a.lengths[(id.sub * a.sg.rows + id.row) * a.sg.nc + id.ch] = len;
+    if (len > a.cap && a.status) atomicOr(a.status, 1);
+}
+
+// ---- decoder (dec_new.cu:35-71, 248-302) -------------------------------------------
+// The decoder tracks off = value - low, which every renormalisation step maps to
+// 2*off + next bit (E1/E2 and E3 alike), and finds the symbol as the largest m with
+// floor(span*cdf[m] / 2^16) <= off; that is the same m as the reference's search of
+// count = ((value-low+1)*2^16 - 1) / span in a strictly increasing table, without the
+// 64-bit divide.  The stream is read through aligned big-endian words with one word of
+// prefetch; bytes past the stream's end read as zero (dec_new.cu:223-233).
+struct BitReader {
+    const uint32_t *words;   // aligned word containing the stream's first byte
+    int64_t nwords_safe;     // words that may be touched
+    uint32_t end_bit;        // first bit (from `words`) past the stream
+    uint32_t w0, w1, w2;
+    int c;                   // unread low bits of w0
+    uint32_t next;           // index of the next word to prefetch
+
+    __device__ __forceinline__ uint32_t load_word(uint32_t j) const
+    {
+        const uint32_t first = j * 32u;
+        uint32_t w = 0;
+        if (first < end_bit) {
+            w = __builtin_bswap32(words[j]);
+            const uint32_t left = end_bit - first;
+            if (left < 32u) w &= 0xFFFFFFFFu << (32u - left);
+        }
+        return w;
+    }
+
+    // position on the stream that starts `skip_bytes` (0..3) into words[0] and is
+    // `len` bytes long; returns its first 32 bits
+    __device__ __forceinline__ uint32_t start(const uint8_t *begin, int len)
+    {
+        const uintptr_t addr = reinterpret_cast<uintptr_t>(begin);
+        const uint32_t skip = (uint32_t)(addr & 3u);
+        words = reinterpret_cast<const uint32_t *>(addr - skip);
+        end_bit = (skip + (uint32_t)len) * 8u;
+        if (skip == 0) {
+            w0 = 0;
+            w1 = load_word(0);
+            w2 = load_word(1);
+            next = 2;
+            c = 0;
+        } else {
+            w0 = load_word(0);
+            w1 = load_word(1);
+            w2 = load_word(2);
+            next = 3;
+            c = 32 - (int)(skip * 8u);
+        }
+        const uint32_t first = __builtin_amdgcn_alignbit(w0, w1, (uint32_t)c);
+        w0 = w1;
+        w1 = w2;
+        w2 = load_word(next++);
+        return first;
+    }
+
+    // off = (off << n) | next n bits, 0 <= n <= 31
+    __device__ __forceinline__ uint32_t shift_in(uint32_t off, int n)
+    {
+        const uint32_t nx = __builtin_amdgcn_alignbit(w0, w1, (uint32_t)c);
+        const uint32_t shifted = __builtin_amdgcn_alignbit(off, nx, (uint32_t)(32 - n));
+        off = n ? shifted : off;
+        c -= n;
+        if (c < 0) {
+            w0 = w1;
+            w1 = w2;
+            c += 32;
+            w2 = load_word(next++);
+        }
+        return off;
+    }
+};
+
+enum { SRC_OFFSETS = 0, SRC_PREFIX = 1, SRC_PADDED = 2 };
+enum { OUT_SYMBOLS = 0, OUT_F16 = 1, OUT_BF16 = 2 };
+
+struct DecodeArgs {
+    const uint16_t *cdf;
+    int32_t lp;
+    const uint8_t *bytes;       // payload, or padded buffer
+    const int64_t *offsets;     // SRC_OFFSETS: exclusive sums [nstreams+1]; SRC_PREFIX: inclusive sums
+    const int32_t *lengths;     // SRC_PADDED
+    int64_t p0, p1;             // SRC_PADDED strides
+    int32_t cap;
+    // OUT_SYMBOLS: out[row*o0 + token*o1 + channel*o2] uint8
+    uint8_t *out_sym;
+    int64_t o0, o1, o2;
+    // OUT_F16 / OUT_BF16: dequantised KV, out[l*ol + kv*okv + token*ot + head*oh + dim]
+    uint16_t *out_kv;
+    int64_t ol, okv, ot, oh;
+    int64_t L;
+    int32_t D;
+    const uint16_t *maxima;     // [2, L, T]
+    int32_t max_dt;
+    const float *key_bins, *value_bins;
+    StreamGrid sg;
+};
+
+template <int SRC, int OUT, int MAXDT>
+__global__ __launch_bounds__(256) void decode_streams_kernel(DecodeArgs a)
+{
+    extern __shared__ uint32_t smem[];
+    const int bs = blockDim.x, tid = threadIdx.x;
+    const StreamId id = locate(a.sg);
+    const int lp = a.lp;
+    uint32_t *tab = smem;
+    float *lut = reinterpret_cast<float *>(smem + lp * bs);   // (s - C) / C per symbol
+    float *rowmax = lut + lp;                                 // one per token of the sub-chunk
+    const int64_t ch0 = id.ch - tid;
+    stage_tables(tab, a.cdf + ((id.chunk * a.sg.rows + id.row) * a.sg.nc + ch0) * lp, lp, ch0, a.sg.nc);
+    int64_t kvi = 0, l = 0;
+    if (OUT != OUT_SYMBOLS) {
+        kvi = id.row / a.L;
+        l = id.row - kvi * a.L;
+        const float bins = (kvi ? a.value_bins : a.key_bins)[l];
+        const float cq = floorf(bins * 0.5f) - 1.0f;
+        for (int i = tid; i < lp; i += bs) lut[i] = __fdiv_rn(__fsub_rn((float)i, cq), cq);
+        const uint16_t *mx = a.maxima + id.row * a.sg.g.T + id.t0;
+        for (int i = tid; i < id.n; i += bs) rowmax[i] = load16f<MAXDT>(mx[i]);
+    }
+    __syncthreads();
+    if (!id.active) return;
+
+    const int64_t stream = (id.sub * a.sg.rows + id.row) * a.sg.nc + id.ch;
+    const uint8_t *begin;
+    int len;
+    if (SRC == SRC_OFFSETS) {
+        const int64_t b0 = a.offsets[stream], b1 = a.offsets[stream + 1];
+        begin = a.bytes + b0;
+        len = (int)(b1 - b0);
+    } else if (SRC == SRC_PREFIX) {
+        const int64_t b0 = stream ? a.offsets[stream - 1] : 0, b1 = a.offsets[stream];
+        begin = a.bytes + b0;
+        len = (int)(b1 - b0);
+    } else {
+        begin = a.bytes + id.row * a.p0 + id.ch * a.p1;
+        len = a.lengths[stream];
+        len = len < a.cap ? len : a.cap;
+    }
+    len = len < 0 ? 0 : len;
+
+    BitReader rd;
+    uint32_t off = rd.start(begin, len);
+    uint32_t low = 0, high = 0xFFFFFFFFu;
+
+    uint8_t *osym = nullptr;
+    uint16_t *okv = nullptr;
+    if (OUT == OUT_SYMBOLS) {
+        osym = a.out_sym + id.row * a.o0 + id.t0 * a.o1 + id.ch * a.o2;
+    } else {
+        const int64_t h = id.ch / a.D;
+        okv = a.out_kv + l * a.ol + kvi * a.okv + id.t0 * a.ot + h * a.oh + (id.ch - h * a.D);
+    }
+
+    int nsteps = 0;
+    while ((1 << nsteps) < lp - 1) ++nsteps;
+    const uint32_t c0 = tab[tid];
+
+    for (int i = 0; i < id.n; ++i) {
+        const uint32_t r = high - low;
+        const uint32_t rh = r >> 16, rl = r & 0xFFFFu;
+        int lo_i = 0, hi_i = lp - 1;
+        uint32_t t_lo = scale16(rh, rl, c0);
+        uint32_t t_hi = r + 1u;                         // table end is 2^16 (dec_new.cu:278)
+        for (int step = 0; step < nsteps; ++step) {
+            const int mid = (lo_i + hi_i) >> 1;
+            const uint32_t t = scale16(rh, rl, tab[mid * bs + tid]);
+            const bool le = t <= off;
+            lo_i = le ? mid : lo_i;
+            t_lo = le ? t : t_lo;
+            hi_i = le ? hi_i : mid;
+            t_hi = le ? t_hi : t;
+        }
+        if (OUT == OUT_SYMBOLS) {
+            osym[(int64_t)i * a.o1] = (uint8_t)lo_i;
+        } else {
+            const float v = __fmul_rn(lut[lo_i], rowmax[i]);
+            okv[(int64_t)i * a.ot] = (uint16_t)(OUT == OUT_BF16 ? store16f<CG_DT_BF16>(v)
+                                                                : store16f<CG_DT_F16>(v));
+        }
+        if (i == id.n - 1) break;                       // no update after the last symbol
+        high = low + t_hi - 1u;
+        low = low + t_lo;
+        off -= t_lo;
+
+        const int n1 = __builtin_clz(low ^ high);
+        const uint32_t lo1 = low << n1;
+        const uint32_t hi1 = (high << n1) | ((1u << n1) - 1u);
+        const int k = __builtin_clz(~((lo1 & ~hi1) << 1));
+        low = (lo1 << k) & 0x7FFFFFFFu;
+        high = (hi1 << k) | 0x80000000u | ((1u << k) - 1u);
+        if (n1 + k <= 31) {
+            off = rd.shift_in(off, n1 + k);
+        } else {
+            off = rd.shift_in(off, n1);
+            off = rd.shift_in(off, k);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------
+// Exclusive running sum of the stream lengths (replaces the cumsum of decoder.py:70 and
+// the index arithmetic of encoder.py:214-221): per-block sums, a one-block scan of
+// those, then a per-block scan with the block's base added.
+// ------------------------------------------------------------------------------------
+constexpr int kScanThreads = 256;
+constexpr int kScanPerThread = 8;
+constexpr int kScanTile = kScanThreads * kScanPerThread;
+
+__device__ __forceinline__ int64_t block_exclusive_scan(int64_t v, int64_t *lds, int64_t &total)
+{
+    const int tid = threadIdx.x;
+    lds[tid] = v;
+    __syncthreads();
+    for (int o = 1; o < kScanThreads; o <<= 1) {
+        const int64_t add = tid >= o ? lds[tid - o] : 0;
+        __syncthreads();
+        lds[tid] += add;
+        __syncthreads();
+    }
+    total = lds[kScanThreads - 1];
+    const int64_t incl = lds[tid];
+    __syncthreads();
+    return incl - v;
+}
+
+__global__ __launch_bounds__(kScanThreads) void scan_tile_sums_kernel(
+    const int32_t *__restrict__ lengths, int64_t n, int32_t clamp, int64_t *__restrict__ sums)
+{
+    __shared__ int64_t lds[kScanThreads];
+    const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanPerThread;
+    int64_t s = 0;
+    for (int j = 0; j < kScanPerThread; ++j)
+        if (base + j < n) {
+            int32_t v = lengths[base + j];
+            v = v < 0 ? 0 : (v > clamp ? clamp : v);
+            s += v;
+        }
+    int64_t total;
+    block_exclusive_scan(s, lds, total);
+    if (threadIdx.x == 0) sums[blockIdx.x] = total;
+}
+
+__global__ __launch_bounds__(kScanThreads) void scan_sums_kernel(int64_t *sums, int64_t ntiles)
+{
+    __shared__ int64_t lds[kScanThreads];
+    int64_t carry = 0;
+    for (int64_t base = 0; base < ntiles; base += kScanThreads) {
+        const int64_t i = base + threadIdx.x;
+        const int64_t v = i < ntiles ? sums[i] : 0;
+        int64_t total;
+        const int64_t ex = block_exclusive_scan(v, lds, total);
+        if (i < ntiles) sums[i] = carry + ex;
+        carry += total;
+    }
+}
+
+__global__ __launch_bounds__(kScanThreads) void scan_apply_kernel(
+    const int32_t *__restrict__ lengths, int64_t n, int32_t clamp,
+    const int64_t *__restrict__ sums, int64_t *__restrict__ offsets)
+{
+    __shared__ int64_t lds[kScanThreads];
+    const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanPerThread;
+    int32_t v[kScanPerThread];
+    int64_t s = 0;
+    for (int j = 0; j < kScanPerThread; ++j) {
+        int32_t x = base + j < n ? lengths[base + j] : 0;
+        x = x < 0 ? 0 : (x > clamp ? clamp : x);
+        v[j] = x;
+        s += x;
+    }
+    int64_t total;
+    int64_t run = sums[blockIdx.x] + block_exclusive_scan(s, lds, total);
+    for (int j = 0; j < kScanPerThread; ++j) {
+        if (base + j < n) offsets[base + j] = run;
+        run += v[j];
+        if (base + j == n - 1) offsets[n] = run;
+    }
+}
+
+// ------------------------------------------------------------------------------------
+// collect_bytes (encoder.py:209-222): each wavefront moves 64 streams from their padded
+// slots to their final offsets, one stream at a time with all lanes copying.
+// ------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void compact_streams_kernel(
+    const uint8_t *__restrict__ padded, int32_t cap, const int32_t *__restrict__ lengths,
+    const int64_t *__restrict__ offsets, int64_t nstreams, uint8_t *__restrict__ payload,
+    int64_t payload_cap, int32_t *status)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t first = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * 64;
+    if (first >= nstreams) return;
+    const int64_t mine = first + lane;
+    int my_len = 0;
+    int64_t my_off = 0;
+    if (mine < nstreams) {
+        my_len = lengths[mine];
+        my_len = my_len < 0 ? 0 : (my_len > cap ? cap : my_len);
+        my_off = offsets[mine];
+    }
+    const int count = (nstreams - first < 64) ? (int)(nstreams - first) : 64;
+    bool spilled = false;
+    for (int s = 0; s < count; ++s) {
+        const int len = __shfl(my_len, s, 64);
+        const int64_t off = __shfl(my_off, s, 64);
+        const uint8_t *src = padded + (first + s) * (int64_t)cap;
+        for (int j = lane; j < len; j += 64) {
+            if (off + j < payload_cap) payload[off + j] = src[j];
+            else spilled = true;
+        }
+    }
+    if (spilled && status) atomicOr(status, 2);
+}
+
+__global__ void clear_status_kernel(int32_t *status) { *status = 0; }
+
+// ------------------------------------------------------------------------------------
+// host-side launch helpers
+// ------------------------------------------------------------------------------------
+// Lanes per block: as many adjacent channels as possible while the per-block table
+// (lp words per lane) stays well inside the default dynamic LDS window.
+int pick_block(int64_t nc, int lp)
+{
+    int block = 256;
+    if (lp > 40) block = 128;
+    if (lp > 80) block = 64;
+    while (block > 64 && nc <= block / 2) block /= 2;
+    return block;
+}
+
+int make_grid(int64_t rows, int64_t nc, int64_t T, int64_t S, int64_t nsub, int block,
+              StreamGrid &sg, int64_t &nblocks)
+{
+    sg.rows = rows;
+    sg.nc = nc;
+    sg.ctiles = (int32_t)ceil_div(nc, block);
+    sg.g.T = T;
+    sg.g.S = S;
+    sg.g.nsc = (int32_t)ceil_div(S, kSub);
+    nblocks = nsub * rows * sg.ctiles;
+    if (nblocks <= 0 || nblocks > INT_MAX) return fail(CG_ERR_ARG, "grid of %lld blocks is out of range", (long long)nblocks);
+    return CG_OK;
+}
+
+int launch_cdf(const uint8_t *sym, int64_t rows, int64_t T, int64_t nc, int64_t s0, int64_t s1,
+               int64_t s2, int max_bins, int64_t S, uint16_t *cdf, hipStream_t stream)
+{
+    const int block = pick_block(nc, max_bins + 1);
+    CdfArgs a;
+    a.sym = sym;
+    a.s0 = s0;
+    a.s1 = s1;
+    a.s2 = s2;
+    a.cdf = cdf;
+    a.rows = rows;
+    a.nc = nc;
+    a.ctiles = (int32_t)ceil_div(nc, block);
+    a.max_bins = max_bins;
+    a.g.T = T;
+    a.g.S = S;
+    a.g.nsc = (int32_t)ceil_div(S, kSub);
+    const int64_t nblocks = ceil_div(T, S) * rows * a.ctiles;
+    if (nblocks <= 0 || nblocks > INT_MAX) return fail(CG_ERR_ARG, "calculate_cdf: grid out of range");
+    const size_t shmem = (size_t)(max_bins + 1) * block * sizeof(uint32_t);
+    calculate_cdf_kernel<<<dim3((unsigned)nblocks), dim3(block), shmem, stream>>>(a);
+    return check_launch("calculate_cdf");
+}
+
+int launch_scan(const int32_t *lengths, int64_t n, int32_t clamp, int64_t *offsets, void *scratch,
+                hipStream_t stream)
+{
+    const int64_t ntiles = ceil_div(n, kScanTile);
+    int64_t *sums = static_cast<int64_t *>(scratch);
+    scan_tile_sums_kernel<<<dim3((unsigned)ntiles), dim3(kScanThreads), 0, stream>>>(lengths, n, clamp, sums);
+    scan_sums_kernel<<<dim3(1), dim3(kScanThreads), 0, stream>>>(sums, ntiles);
+    scan_apply_kernel<<<dim3((unsigned)ntiles), dim3(kScanThreads), 0, stream>>>(lengths, n, clamp, sums, offsets);
+    return check_launch("scan_lengths");
+}
+
+int check_dt(int dt, const char *what)
+{
+    if (dt != CG_DT_F16 && dt != CG_DT_BF16) return fail(CG_ERR_ARG, "%s: dtype must be CG_DT_F16 or CG_DT_BF16", what);
+    return CG_OK;
+}
+
+int check_lp(int lp, const char *what)
+{
+    if (lp < 2 || lp > CG_MAX_LP) return fail(CG_ERR_ARG, "%s: CDF length should be in [2, %d], got %d", what, CG_MAX_LP, lp);
+    return CG_OK;
+}
+
+int launch_quantize(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D,
+                    int64_t sl, int64_t skv, int64_t st, int64_t sh, const float *key_bins,
+                    const float *value_bins, uint8_t *sym, void *maxima, hipStream_t stream)
+{
+    const int64_t C = H * D;
+    const int64_t nrows = 2 * L * T;
+    const int64_t nblocks = ceil_div(nrows, 4);
+    if (nblocks > INT_MAX || C > INT_MAX) return fail(CG_ERR_ARG, "quantize: tensor too large for one launch");
+    const bool vec = (D % 8 == 0) && (sl % 8 == 0) && (skv % 8 == 0) && (st % 8 == 0) && (sh % 8 == 0) &&
+                     aligned_to(kv, 16) && aligned_to(sym, 8) && (C / 8 <= 64 * kMaxUnits);
+    const uint16_t *p = static_cast<const uint16_t *>(kv);
+    uint16_t *mx = static_cast<uint16_t *>(maxima);
+    dim3 grid((unsigned)nblocks), block(256);
+    if (vec) {
+        const int nunits = (int)(C / 8);
+        const bool contiguous = (sh == D);
+#define CG_LAUNCH_Q(DT, HC) quantize_kv_kernel<DT, HC><<<grid, block, 0, stream>>>( \
+        p, L, T, (int)D, sl, skv, st, sh, key_bins, value_bins, sym, mx, nunits, nrows)
+        if (kv_dt == CG_DT_F16) { if (contiguous) CG_LAUNCH_Q(CG_DT_F16, true); else CG_LAUNCH_Q(CG_DT_F16, false); }
+        else { if (contiguous) CG_LAUNCH_Q(CG_DT_BF16, true); else CG_LAUNCH_Q(CG_DT_BF16, false); }
+#undef CG_LAUNCH_Q
+    } else {
+        if (kv_dt == CG_DT_F16)
+            quantize_kv_generic_kernel<CG_DT_F16><<<grid, block, 0, stream>>>(
+                p, L, T, (int)D, (int)C, sl, skv, st, sh, key_bins, value_bins, sym, mx, nrows);
+        else
+            quantize_kv_generic_kernel<CG_DT_BF16><<<grid, block, 0, stream>>>(
+                p, L, T, (int)D, (int)C, sl, skv, st, sh, key_bins, value_bins, sym, mx, nrows);
+    }
+    return check_launch("quantize_kv");
+}
+
+template <int SRC, int OUT>
+int launch_decode_dt(const DecodeArgs &a, int64_t nblocks, int block, size_t shmem, hipStream_t stream)
+{
+    if (a.max_dt == CG_DT_BF16)
+        decode_streams_kernel<SRC, OUT, CG_DT_BF16><<<dim3((unsigned)nblocks), dim3(block), shmem, stream>>>(a);
+    else
+        decode_streams_kernel<SRC, OUT, CG_DT_F16><<<dim3((unsigned)nblocks), dim3(block), shmem, stream>>>(a);
+    return check_launch("decode");
+}
+
+}  // namespace
+
+// ======================================================================================
+// C ABI
+// ======================================================================================
+extern "C" {
+
+const char *cg_last_error(void) { return g_error; }
+int cg_abi_version(void) { return 1; }
+
+int64_t cg_num_chunks(int64_t T, int64_t chunk_tokens)
+{
+    if (T <= 0 || chunk_tokens <= 0) return 0;
+    return ceil_div(T, chunk_tokens);
+}
+
+int64_t cg_num_subchunks(int64_t T, int64_t chunk_tokens)
+{
+    if (T <= 0 || chunk_tokens <= 0) return 0;
+    const int64_t nchunks = ceil_div(T, chunk_tokens);
+    const int64_t last = T - (nchunks - 1) * chunk_tokens;
+    return (nchunks - 1) * ceil_div(chunk_tokens, kSub) + ceil_div(last, kSub);
+}
+
+int cg_calculate_cdf(const int8_t *sym, int64_t nl, int64_t nt, int64_t nc, int64_t s0, int64_t s1,
+                     int64_t s2, int max_bins, int16_t *cdf, void *stream)
+{
+    if (!sym || !cdf) return fail(CG_ERR_ARG, "calculate_cdf: null pointer");
+    if (nl <= 0 || nt <= 0 || nc <= 0) return fail(CG_ERR_ARG, "calculate_cdf: empty input");
+    if (max_bins < 1 || max_bins + 1 > CG_MAX_LP) return fail(CG_ERR_ARG, "Max bins must be less than %d", CG_MAX_LP);
+    if (nt > 65535) return fail(CG_ERR_ARG, "calculate_cdf: at most 65535 tokens per table (16-bit counters)");
+    return launch_cdf(reinterpret_cast<const uint8_t *>(sym), nl, nt, nc, s0, s1, s2, max_bins, nt,
+                      reinterpret_cast<uint16_t *>(cdf), static_cast<hipStream_t>(stream));
+}
+
+int cg_encode_fast_new(const int16_t *cdf, int lp, const int8_t *sym, int64_t nl, int64_t nt, int64_t nc,
+                       int64_t s0, int64_t s1, int64_t s2, uint8_t *out, int64_t cap, int64_t o0,
+                       int64_t o1, int32_t *lengths, void *stream)
+{
+    if (!cdf || !sym || !out || !lengths) return fail(CG_ERR_ARG, "encode: null pointer");
+    if (int rc = check_lp(lp, "encode")) return rc;
+    if (nl <= 0 || nc <= 0 || nt < 0) return fail(CG_ERR_ARG, "encode: empty input");
+    if (nt > kSub) return fail(CG_ERR_ARG, "Number of tokens should be less than or equal to %d", kSub);
+    if (cap <= 0 || cap > INT_MAX) return fail(CG_ERR_ARG, "encode: bad output buffer length");
+    const int block = pick_block(nc, lp);
+    EncodeArgs a;
+    a.cdf = reinterpret_cast<const uint16_t *>(cdf);
+    a.lp = lp;
+    a.sym = reinterpret_cast<const uint8_t *>(sym);
+    a.s0 = s0;
+    a.s1 = s1;
+    a.s2 = s2;
+    a.out = out;
+    a.osub = 0;
+    a.o0 = o0;
+    a.o1 = o1;
+    a.cap = (int32_t)cap;
+    a.lengths = lengths;
+    a.status = nullptr;
+    int64_t nblocks;
+    // nt == 0 still writes the two tail bits of every stream
+    if (int rc = make_grid(nl, nc, nt ? nt : 1, nt ? nt : 1, 1, block, a.sg, nblocks)) return rc;
+    if (nt == 0) a.sg.g.T = 0;
+    const size_t shmem = (size_t)lp * block * sizeof(uint32_t);
+    const bool aligned = aligned_to(out, 4) && o0 % 4 == 0 && o1 % 4 == 0;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (aligned) encode_streams_kernel<true><<<dim3((unsigned)nblocks), dim3(block), shmem, st>>>(a);
+    else encode_streams_kernel<false><<<dim3((unsigned)nblocks), dim3(block), shmem, st>>>(a);
+    return check_launch("encode");
+}
+
+int cg_decode_fast_new(const int16_t *cdf, int lp, const uint8_t *padded, int64_t cap, int64_t p0,
+                       int64_t p1, const int32_t *lengths, int64_t nl, int64_t nt, int64_t nc,
+                       uint8_t *out, int64_t o0, int64_t o1, int64_t o2, void *stream)
+{
+    if (!cdf || !padded || !lengths || !out) return fail(CG_ERR_ARG, "decode: null pointer");
+    if (int rc = check_lp(lp, "decode")) return rc;
+    if (nl <= 0 || nc <= 0 || nt <= 0) return fail(CG_ERR_ARG, "decode: empty input");
+    if (nt > kSub) return fail(CG_ERR_ARG, "Number of tokens should be less than or equal to %d", kSub);
+    if (cap <= 0 || cap > INT_MAX) return fail(CG_ERR_ARG, "decode: bad padded buffer length");
+    const int block = pick_block(nc, lp);
+    DecodeArgs a;
+    memset(&a, 0, sizeof(a));
+    a.cdf = reinterpret_cast<const uint16_t *>(cdf);
+    a.lp = lp;
+    a.bytes = padded;
+    a.lengths = lengths;
+    a.p0 = p0;
+    a.p1 = p1;
+    a.cap = (int32_t)cap;
+    a.out_sym = out;
+    a.o0 = o0;
+    a.o1 = o1;
+    a.o2 = o2;
+    int64_t nblocks;
+    if (int rc = make_grid(nl, nc, nt, nt, 1, block, a.sg, nblocks)) return rc;
+    const size_t shmem = (size_t)lp * block * sizeof(uint32_t) + (lp + kSub) * sizeof(float);
+    return launch_decode_dt<SRC_PADDED, OUT_SYMBOLS>(a, nblocks, block, shmem, static_cast<hipStream_t>(stream));
+}
+
+int cg_decode_fast_prefsum(const int16_t *cdf, int lp, const uint8_t *bytes, int64_t nbytes,
+                           const int64_t *prefix, int64_t nl, int64_t nt, int64_t nc, uint8_t *out,
+                           int64_t o0, int64_t o1, int64_t o2, void *stream)
+{
+    if (!cdf || !prefix || !out || (!bytes && nbytes > 0)) return fail(CG_ERR_ARG, "decode: null pointer");
+    if (int rc = check_lp(lp, "decode")) return rc;
+    if (nl <= 0 || nc <= 0 || nt <= 0) return fail(CG_ERR_ARG, "decode: empty input");
+    if (nt > kSub) return fail(CG_ERR_ARG, "Number of tokens should be less than or equal to %d", kSub);
+    const int block = pick_block(nc, lp);
+    DecodeArgs a;
+    memset(&a, 0, sizeof(a));
+    a.cdf = reinterpret_cast<const uint16_t *>(cdf);
+    a.lp = lp;
+    a.bytes = bytes;
+    a.offsets = prefix;
+    a.out_sym = out;
+    a.o0 = o0;
+    a.o1 = o1;
+    a.o2 = o2;
+    int64_t nblocks;
+    if (int rc = make_grid(nl, nc, nt, nt, 1, block, a.sg, nblocks)) return rc;
+    const size_t shmem = (size_t)lp * block * sizeof(uint32_t) + (lp + kSub) * sizeof(float);
+    return launch_decode_dt<SRC_PREFIX, OUT_SYMBOLS>(a, nblocks, block, shmem, static_cast<hipStream_t>(stream));
+}
+
+int cg_quantize_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D, int64_t sl,
+                   int64_t skv, int64_t st, int64_t sh, const float *key_bins, const float *value_bins,
+                   uint8_t *sym, void *maxima, void *stream)
+{
+    if (!kv || !key_bins || !value_bins || !sym || !maxima) return fail(CG_ERR_ARG, "quantize: null pointer");
+    if (int rc = check_dt(kv_dt, "quantize")) return rc;
+    if (L <= 0 || T <= 0 || H <= 0 || D <= 0) return fail(CG_ERR_ARG, "quantize: empty input");
+    return launch_quantize(kv, kv_dt, L, T, H, D, sl, skv, st, sh, key_bins, value_bins, sym, maxima,
+                           static_cast<hipStream_t>(stream));
+}
+
+size_t cg_scan_workspace(int64_t n) { return align_up((size_t)(ceil_div(n > 0 ? n : 1, kScanTile) + 1) * sizeof(int64_t), 256); }
+
+int cg_scan_lengths(const int32_t *lengths, int64_t n, int64_t *offsets, void *scratch,
+                    size_t scratch_bytes, void *stream)
+{
+    if (!lengths || !offsets || !scratch) return fail(CG_ERR_ARG, "scan: null pointer");
+    if (n <= 0) return fail(CG_ERR_ARG, "scan: empty input");
+    if (scratch_bytes < cg_scan_workspace(n)) return fail(CG_ERR_WORKSPACE, "scan: scratch too small");
+    return launch_scan(lengths, n, INT_MAX, offsets, scratch, static_cast<hipStream_t>(stream));
+}
+
+size_t cg_encode_kv_workspace(int64_t L, int64_t T, int64_t C, int64_t chunk_tokens)
+{
+    const int64_t nsub = cg_num_subchunks(T, chunk_tokens);
+    const int64_t nstreams = nsub * 2 * L * C;
+    size_t total = align_up((size_t)(2 * L * T * C), 256);        // symbols
+    total += align_up((size_t)nstreams * kStreamCap, 256);        // padded streams
+    total += cg_scan_workspace(nstreams);
+    return total;
+}
+
+int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D, int64_t sl,
+                 int64_t skv, int64_t st, int64_t sh, const float *key_bins, const float *value_bins,
+                 int max_bins, int64_t chunk_tokens, int16_t *cdf, void *maxima, int32_t *lengths,
+                 int64_t *offsets, uint8_t *payload, int64_t payload_cap, int32_t *status,
+                 void *workspace, size_t workspace_bytes, void *stream)
+{
+    if (!kv || !key_bins || !value_bins || !cdf || !maxima || !lengths || !offsets || !payload || !status || !workspace)
+        return fail(CG_ERR_ARG, "encode_kv: null pointer");
+    if (int rc = check_dt(kv_dt, "encode_kv")) return rc;
+    if (L <= 0 || T <= 0 || H <= 0 || D <= 0) return fail(CG_ERR_ARG, "encode_kv: empty input");
+    if (chunk_tokens <= 0) return fail(CG_ERR_ARG, "encode_kv: chunk_tokens must be positive");
+    if (chunk_tokens > 65535) return fail(CG_ERR_ARG, "encode_kv: at most 65535 tokens per chunk (16-bit counters)");
+    if (int rc = check_lp(max_bins + 1, "encode_kv")) return rc;
+    const int64_t C = H * D, rows = 2 * L;
+    const int64_t nsub = cg_num_subchunks(T, chunk_tokens);
+    const int64_t nstreams = nsub * rows * C;
+    if (workspace_bytes < cg_encode_kv_workspace(L, T, C, chunk_tokens)) return fail(CG_ERR_WORKSPACE, "encode_kv: workspace too small");
+    if (!aligned_to(workspace, 256)) return fail(CG_ERR_ARG, "encode_kv: workspace must be 256-byte aligned");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+
+    uint8_t *ws = static_cast<uint8_t *>(workspace);
+    uint8_t *sym = ws;
+    ws += align_up((size_t)(rows * T * C), 256);
+    uint8_t *padded = ws;
+    ws += align_up((size_t)nstreams * kStreamCap, 256);
+    void *scan_scratch = ws;
+
+    clear_status_kernel<<<1, 1, 0, s>>>(status);
+    if (int rc = launch_quantize(kv, kv_dt, L, T, H, D, sl, skv, st, sh, key_bins, value_bins, sym, maxima, s)) return rc;
+    if (int rc = launch_cdf(sym, rows, T, C, T * C, C, 1, max_bins, chunk_tokens, reinterpret_cast<uint16_t *>(cdf), s)) return rc;
+
+    const int block = pick_block(C, max_bins + 1);
+    EncodeArgs a;
+    a.cdf = reinterpret_cast<const uint16_t *>(cdf);
+    a.lp = max_bins + 1;
+    a.sym = sym;
+    a.s0 = T * C;
+    a.s1 = C;
+    a.s2 = 1;
+    a.out = padded;
+    a.osub = rows * C * kStreamCap;
+    a.o0 = C * kStreamCap;
+    a.o1 = kStreamCap;
+    a.cap = kStreamCap;
+    a.lengths = lengths;
+    a.status = status;
+    int64_t nblocks;
+    if (int rc = make_grid(rows, C, T, chunk_tokens, nsub, block, a.sg, nblocks)) return rc;
+    const size_t shmem = (size_t)a.lp * block * sizeof(uint32_t);
+    encode_streams_kernel<true><<<dim3((unsigned)nblocks), dim3(block), shmem, s>>>(a);
+    if (int rc = check_launch("encode_kv")) return rc;
+
+    if (int rc = launch_scan(lengths, nstreams, kStreamCap, offsets, scan_scratch, s)) return rc;
+    const int64_t cblocks = ceil_div(nstreams, 256);
+    if (cblocks > INT_MAX) return fail(CG_ERR_ARG, "encode_kv: too many streams");
+    compact_streams_kernel<<<dim3((unsigned)cblocks), dim3(256), 0, s>>>(padded, kStreamCap, lengths, offsets,
+                                                                      nstreams, payload, payload_cap, status);
+    return check_launch("compact");
+}
+
+int cg_decode_kv(const int16_t *cdf, int max_bins, const void *maxima, int max_dt, const int64_t *offsets,
+                 const uint8_t *payload, int64_t payload_bytes, const float *key_bins,
+                 const float *value_bins, int64_t L, int64_t T, int64_t H, int64_t D,
+                 int64_t chunk_tokens, void *out, int out_dt, int64_t ol, int64_t okv, int64_t ot,
+                 int64_t oh, void *stream)
+{
+    if (!cdf || !maxima || !offsets || !key_bins || !value_bins || !out || (!payload && payload_bytes > 0))
+        return fail(CG_ERR_ARG, "decode_kv: null pointer");
+    if (int rc = check_dt(max_dt, "decode_kv")) return rc;
+    if (int rc = check_dt(out_dt, "decode_kv")) return rc;
+    if (L <= 0 || T <= 0 || H <= 0 || D <= 0 || chunk_tokens <= 0) return fail(CG_ERR_ARG, "decode_kv: empty input");
+    if (int rc = check_lp(max_bins + 1, "decode_kv")) return rc;
+    const int64_t C = H * D, rows = 2 * L;
+    if (D > INT_MAX) return fail(CG_ERR_ARG, "decode_kv: head size too large");
+    const int64_t nsub = cg_num_subchunks(T, chunk_tokens);
+    const int block = pick_block(C, max_bins + 1);
+    DecodeArgs a;
+    memset(&a, 0, sizeof(a));
+    a.cdf = reinterpret_cast<const uint16_t *>(cdf);
+    a.lp = max_bins + 1;
+    a.bytes = payload;
+    a.offsets = offsets;
+    a.out_kv = static_cast<uint16_t *>(out);
+    a.ol = ol;
+    a.okv = okv;
+    a.ot = ot;
+    a.oh = oh;
+    a.L = L;
+    a.D = (int32_t)D;
+    a.maxima = static_cast<const uint16_t *>(maxima);
+    a.max_dt = max_dt;
+    a.key_bins = key_bins;
+    a.value_bins = value_bins;
+    int64_t nblocks;
+    if (int rc = make_grid(rows, C, T, chunk_tokens, nsub, block, a.sg, nblocks)) return rc;
+    const size_t shmem = (size_t)a.lp * block * sizeof(uint32_t) + (a.lp + kSub) * sizeof(float);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (out_dt == CG_DT_BF16) return launch_decode_dt<SRC_OFFSETS, OUT_BF16>(a, nblocks, block, shmem, s);
+    return launch_decode_dt<SRC_OFFSETS, OUT_F16>(a, nblocks, block, shmem, s);
+}
+
+}  // extern "C"

@@ -1,0 +1,164 @@
+/*
+ * cachegen_hip.h -- C ABI of the MI355X (gfx950) CacheGen KV codec library.
+ *
+ * Plain pointers and sizes only; every pointer named "device" must be memory the
+ * GPU can access, `stream` is a hipStream_t passed as void* (NULL = the null
+ * stream).  All functions are asynchronous with respect to the host, keep no
+ * state between calls and return CG_OK or a negative CG_ERR_* code;
+ * cg_last_error() then holds a message for the calling thread.
+ *
+ * Paths in the comments are relative to LMCache/ in the reference tree:
+ *   enc_new.cu = third_party/torchac_cuda/torchac_kernel_enc_new.cu
+ *   dec_new.cu = third_party/torchac_cuda/torchac_kernel_dec_new.cu
+ *   cal_cdf.cu = third_party/torchac_cuda/cal_cdf.cu
+ *   main.cpp   = third_party/torchac_cuda/main.cpp
+ *   encoder.py = lmcache/storage_backend/serde/cachegen_encoder.py
+ *   decoder.py = lmcache/storage_backend/serde/cachegen_decoder.py
+ */
+#ifndef CACHEGEN_HIP_H
+#define CACHEGEN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CG_OK 0
+#define CG_ERR_ARG (-1)      /* bad shape, stride, dtype or limit */
+#define CG_ERR_LAUNCH (-2)   /* the HIP runtime refused a launch */
+#define CG_ERR_WORKSPACE (-3)/* workspace too small */
+
+#define CG_DT_F16 0
+#define CG_DT_BF16 1
+
+#define CG_MAX_TOKENS_PER_STREAM 256 /* cachegen_basics.py:8, enc_new.cu:9-15 */
+#define CG_MAX_LP 129                /* table length limit of this library (reference: 48 / 64) */
+
+/* Message for the last error returned on this thread ("" if none). */
+const char *cg_last_error(void);
+/* ABI version of the library: bumped when a signature changes. */
+int cg_abi_version(void);
+
+/* ---------------------------------------------------------------------------
+ * The four entry points of the reference's extension module (main.cpp:14-17).
+ * Strides are in elements.  Tables are int16 bit patterns of uint16 values.
+ * ------------------------------------------------------------------------- */
+
+/* torchac_cuda.calculate_cdf (cal_cdf.cu:68-129).
+ * sym  device int8  [nl, nt, nc], strides (s0, s1, s2), values in [0, max_bins)
+ * cdf  device int16 [nl, nc, max_bins + 1], contiguous, written
+ * Counters are 16 bits wide as in the reference, so nt <= 65535 is required. */
+int cg_calculate_cdf(const int8_t *sym, int64_t nl, int64_t nt, int64_t nc,
+                     int64_t s0, int64_t s1, int64_t s2, int max_bins,
+                     int16_t *cdf, void *stream);
+
+/* torchac_cuda.encode_fast_new (enc_new.cu:355-451).
+ * cdf      device int16 [nl, nc, lp] contiguous
+ * sym      device int8  [nl, nt, nc], strides (s0, s1, s2), nt <= 256
+ * out      device uint8 [nl, nc, cap], strides (o0, o1, 1); stream (l, c) is written
+ *          to out[l, c, 0:length]; bytes past the length are left untouched
+ * lengths  device int32 [nl, nc] contiguous, written.  A stream longer than `cap`
+ *          is truncated to `cap` stored bytes while its full length is reported. */
+int cg_encode_fast_new(const int16_t *cdf, int lp, const int8_t *sym,
+                       int64_t nl, int64_t nt, int64_t nc,
+                       int64_t s0, int64_t s1, int64_t s2,
+                       uint8_t *out, int64_t cap, int64_t o0, int64_t o1,
+                       int32_t *lengths, void *stream);
+
+/* torchac_cuda.decode_fast_new (dec_new.cu:314-393): streams in a padded buffer.
+ * padded   device uint8 [nl, nc, cap], strides (p0, p1, 1)
+ * lengths  device int32 [nl, nc] contiguous
+ * out      device uint8 [nl, nt, nc], strides (o0, o1, o2), written */
+int cg_decode_fast_new(const int16_t *cdf, int lp, const uint8_t *padded, int64_t cap,
+                       int64_t p0, int64_t p1, const int32_t *lengths,
+                       int64_t nl, int64_t nt, int64_t nc,
+                       uint8_t *out, int64_t o0, int64_t o1, int64_t o2, void *stream);
+
+/* torchac_cuda.decode_fast_prefsum (dec_new.cu:403-479): streams concatenated in
+ * (layer, channel) order.
+ * bytes    device uint8 [nbytes]
+ * prefix   device int64 [nl, nc] contiguous: INCLUSIVE running sum of the stream
+ *          lengths (decoder.py:70); stream g = l*nc + c is bytes[prefix[g-1]:prefix[g]] */
+int cg_decode_fast_prefsum(const int16_t *cdf, int lp, const uint8_t *bytes, int64_t nbytes,
+                           const int64_t *prefix, int64_t nl, int64_t nt, int64_t nc,
+                           uint8_t *out, int64_t o0, int64_t o1, int64_t o2, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * Fused forms of the Python-side tensor code around those kernels.
+ *
+ * A KV cache is a 16-bit float tensor indexed (layer, k|v, token, head, dim) with
+ * element strides (sl, skv, st, sh, 1): [L,2,T,H,D] ("vllm") and [L,2,H,T,D]
+ * ("huggingface") are both expressible (encoder.py:341-342, decoder.py:169-173).
+ * C = H*D channels; "2L" rows are the L key layers followed by the L value layers
+ * (encoder.py:263).  Tokens are cut into chunks of `chunk_tokens` (one table per
+ * chunk, layer and channel: one `to_bytes` call of the reference each) and every
+ * chunk into sub-chunks of at most 256 tokens (encoder.py:279-292); sub-chunks
+ * are numbered consecutively over the whole tensor (nsub of them).  A stream is
+ * one (sub-chunk, row of 2L, channel), numbered in that order.
+ * ------------------------------------------------------------------------- */
+
+/* torch_quant_vectorized on K and V (encoder.py:42-59, 72-83, 258-263).
+ * kv          device fp16/bf16 KV cache (kv_dt, strides above)
+ * key_bins    device float32 [L], value_bins likewise (encoder.py:311-322)
+ * sym         device uint8 [2L, T, C] contiguous, written
+ * maxima      device 16-bit [2, L, T] contiguous in kv_dt, written: row maxima,
+ *             maxima[0] = max_tensors_key, maxima[1] = max_tensors_value */
+int cg_quantize_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D,
+                   int64_t sl, int64_t skv, int64_t st, int64_t sh,
+                   const float *key_bins, const float *value_bins,
+                   uint8_t *sym, void *maxima, void *stream);
+
+/* Number of sub-chunks / chunks for T tokens cut every chunk_tokens. */
+int64_t cg_num_chunks(int64_t T, int64_t chunk_tokens);
+int64_t cg_num_subchunks(int64_t T, int64_t chunk_tokens);
+
+/* Bytes of device workspace cg_encode_kv needs. */
+size_t cg_encode_kv_workspace(int64_t L, int64_t T, int64_t C, int64_t chunk_tokens);
+
+/* encode_function for every chunk at once (encoder.py:247-301), including
+ * collect_bytes (encoder.py:209-222).
+ * cdf         device int16 [nchunks, 2L, C, max_bins+1], written
+ * maxima      device 16-bit [2, L, T] in kv_dt, written
+ * lengths     device int32 [nsub, 2L, C], written: bytes of every stream
+ * offsets     device int64 [nsub*2L*C + 1], written: exclusive running sum of the
+ *             lengths; offsets[last] = total payload bytes
+ * payload     device uint8 [payload_cap], written: all streams back to back in
+ *             stream order; the streams of sub-chunk g are
+ *             payload[offsets[g*2L*C] : offsets[(g+1)*2L*C]] = that sub-chunk's
+ *             `bytestream` tensor.  payload_cap >= 256 * number of streams is
+ *             always enough.
+ * status      device int32 [1], written: 0, or 1 if a stream exceeded 256 bytes
+ *             (the reference overruns its buffer there; here the stream is cut).
+ * workspace   device scratch of cg_encode_kv_workspace(...) bytes, 256-aligned */
+int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D,
+                 int64_t sl, int64_t skv, int64_t st, int64_t sh,
+                 const float *key_bins, const float *value_bins, int max_bins,
+                 int64_t chunk_tokens,
+                 int16_t *cdf, void *maxima, int32_t *lengths, int64_t *offsets,
+                 uint8_t *payload, int64_t payload_cap, int32_t *status,
+                 void *workspace, size_t workspace_bytes, void *stream);
+
+/* Exclusive running sum of stream lengths: offsets[0] = 0, offsets[i+1] =
+ * offsets[i] + lengths[i] (the inclusive sums of decoder.py:70 are offsets[1:]).
+ * scratch: device, cg_scan_workspace(n) bytes. */
+size_t cg_scan_workspace(int64_t n);
+int cg_scan_lengths(const int32_t *lengths, int64_t n, int64_t *offsets,
+                    void *scratch, size_t scratch_bytes, void *stream);
+
+/* decode_function_gpu + do_dequantize + the final cast and layout (decoder.py:
+ * 77-112, 24-34, 159-173) for every chunk at once.
+ * cdf, maxima, offsets, payload: as written by cg_encode_kv (maxima in max_dt)
+ * out         device fp16/bf16 KV cache (out_dt, strides (ol, okv, ot, oh, 1)), written */
+int cg_decode_kv(const int16_t *cdf, int max_bins, const void *maxima, int max_dt,
+                 const int64_t *offsets, const uint8_t *payload, int64_t payload_bytes,
+                 const float *key_bins, const float *value_bins,
+                 int64_t L, int64_t T, int64_t H, int64_t D, int64_t chunk_tokens,
+                 void *out, int out_dt, int64_t ol, int64_t okv, int64_t ot, int64_t oh,
+                 void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CACHEGEN_HIP_H */

@@ -1,0 +1,199 @@
+#!/usr/bin/env python3
+"""Benchmark of the KV codec hot path on one MI355X.
+
+A step is one encode of the whole synthetic KV cache followed by one decode of the
+result, inputs and outputs resident in HBM, every buffer allocated before the timed
+region.  Prints ONE JSON line.  Workload (default): the Mistral-7B-shape cache of
+BASELINE.json configs[1]: 32 layers x {K,V} x 8192 tokens x 8 heads x 128, fp16, one
+table per 256-token chunk, reference 7B bins table.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+WORKLOADS = {
+    # name: (layers, tokens, heads, head_size, chunk_tokens, model name for the bins table, seed)
+    "config1": (2, 512, 8, 64, 512, None, 1235),
+    "config2": (32, 8192, 8, 128, 256, "mistralai/Mistral-7B-Instruct-v0.2", 1236),
+    "config2_small": (32, 1024, 8, 128, 256, "mistralai/Mistral-7B-Instruct-v0.2", 1236),
+}
+
+
+def bins_for(name, model, layers):
+    import torch
+    from cachegen_amd.serde import cachegen_basics as B
+    if model is None:        # config 1: 32 bins for the first half of the layers, 16 for the rest
+        k = torch.tensor([32.0] * (layers // 2) + [16.0] * (layers - layers // 2))
+        return k, k.clone()
+    os.environ.setdefault("QUANT_LEVEL", "2")
+    cfg = B.CacheGenConfig.from_model_name(model)
+    return B.make_key_bins(cfg), B.make_value_bins(cfg)
+
+
+def algorithmic_bytes(L, T, C, lp, nchunks, nstreams, payload):
+    """Bytes that must cross HBM: the 16-bit tensor once, the compact payload once, the tables,
+    one int32 length per stream and the row maxima."""
+    n = 2 * L * T * C
+    side = 2 * lp * (2 * L * C) * nchunks + 4 * nstreams + 2 * 2 * L * T
+    return dict(kv=2 * n, side=side, payload=payload, encode=2 * n + payload + side,
+                decode=2 * n + payload + side)
+
+
+def cpu_baseline(kv_cpu, kbins, vbins, chunk, sample_tokens):
+    """The oracle's CPU path (C, OpenMP over streams) on the first `sample_tokens` tokens."""
+    import numpy as np
+    import torch
+    from oracle import cachegen_oracle as oracle
+    L, _, T, H, D = kv_cpu.shape
+    n = min(sample_tokens, T)
+    flat = kv_cpu[:, :, :n].reshape(L, 2, n, H * D).contiguous().view(torch.int16).numpy().view(np.uint16)
+    kb, vb = kbins.numpy(), vbins.numpy()
+    oracle.lib()
+    cores = oracle.max_threads()
+    t0 = time.perf_counter()
+    encs = [oracle.encode_function(flat[:, :, s:min(s + chunk, n)], kb, vb) for s in range(0, n, chunk)]
+    t1 = time.perf_counter()
+    for e in encs:
+        oracle.decode_function(e, kb, vb)
+    t2 = time.perf_counter()
+    nbytes = 2 * L * n * H * D * 2
+    return dict(value=round(2 * nbytes / (t2 - t0) / 1e9, 4), unit="GB/s", cores=cores, kind="port",
+                sample="first %d tokens of the workload (%d chunks of %d): %.1f MB fp16, C oracle with OpenMP"
+                       % (n, len(encs), chunk, nbytes / 1e6),
+                encode_GBps=round(nbytes / (t1 - t0) / 1e9, 4), decode_GBps=round(nbytes / (t2 - t1) / 1e9, 4))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="config2", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-sample-tokens", type=int, default=1024)
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this codec runs on one GPU; --gpus must be 1 (the path shards by layer or by "
+              "token chunk with no exchange, see DESIGN.md)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from cachegen_amd import codec
+    from cachegen_amd.kvgen import make_kv
+
+    L, T, H, D, chunk, model, seed = WORKLOADS[args.workload]
+    C = H * D
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    kbins, vbins = bins_for(args.workload, model, L)
+    kv = make_kv(L, T, H, D, seed=seed, device=dev)
+    kb, vb = kbins.to(dev), vbins.to(dev)
+    max_bins = int(max(kbins.max(), vbins.max()))
+
+    workspace = torch.empty(codec.encode_workspace_bytes(L, T, C, chunk), dtype=torch.uint8, device=dev)
+    enc = codec.encode_kv(kv, kb, vb, chunk_tokens=chunk, max_bins=max_bins, workspace=workspace)
+    enc.check()
+    out = torch.empty((L, 2, T, H, D), dtype=torch.float16, device=dev)
+
+    def encode():
+        codec.encode_kv(kv, kb, vb, chunk_tokens=chunk, max_bins=max_bins, workspace=workspace, out=enc)
+
+    def decode():
+        codec.decode_encoded(enc, kb, vb, fmt="vllm", out=out)
+
+    for _ in range(args.warmup):
+        encode()
+        decode()
+    torch.cuda.synchronize()
+
+    # per-phase device times: HIP events on the stream the kernels are queued on
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        ev[i][0].record()
+        encode()
+        ev[i][1].record()
+        decode()                      # a single launch of decode_streams_kernel
+        ev[i][2].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    enc_ms = sorted(e[0].elapsed_time(e[1]) for e in ev)
+    dec_ms = sorted(e[1].elapsed_time(e[2]) for e in ev)
+    enc_avg = sum(enc_ms) / len(enc_ms)
+    dec_avg = sum(dec_ms) / len(dec_ms)
+    ms_per_step = wall * 1000.0 / args.steps
+
+    enc.check()
+    payload = enc.total_bytes()
+    nstreams = enc.lengths.numel()
+    ab = algorithmic_bytes(L, T, C, max_bins + 1, enc.num_chunks, nstreams, payload)
+    kv_bytes = ab["kv"]
+
+    # round trip must reconstruct within half a quantization step of every row
+    x = kv.view(L, 2, T, C).float()
+    y = out.view(L, 2, T, C).float()
+    maxq = torch.stack([kb, vb], dim=1).div(2, rounding_mode="floor").sub(1)[:, :, None, None]
+    step = x.abs().amax(dim=-1, keepdim=True) / maxq
+    verified = bool(((x - y).abs() <= 0.52 * step).all())   # half a step + the 16-bit rounding of the output
+    del x, y
+
+    result = {
+        "metric": "KV encode & decode GB/s (fp16 input) + % HBM roofline + compression ratio",
+        "value": round(2 * kv_bytes / (ms_per_step * 1e-3) / 1e9, 3),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u32",
+        "data": "synthetic",
+        "config": {
+            "workload": "%s: %d layers x {K,V} x %d tokens x %d heads x %d, fp16, one table per %d tokens, "
+                        "AR(1) rho=0.9 lognormal-channel generator seed %d" % (args.workload, L, T, H, D, chunk, seed),
+            "value_is": "fp16 KV bytes encoded plus decoded per second of a full encode+decode step",
+            "kv_bytes": kv_bytes,
+            "streams": nstreams,
+        },
+        "encode_GBps": round(kv_bytes / (enc_avg * 1e-3) / 1e9, 3),
+        "decode_GBps": round(kv_bytes / (dec_avg * 1e-3) / 1e9, 3),
+        "encode_ms": round(enc_avg, 4),
+        "decode_ms": round(dec_avg, 4),
+        "encode_roofline_frac": round(ab["encode"] / (enc_avg * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+        "decode_roofline_frac": round(ab["decode"] / (dec_avg * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+        "compression_ratio_payload": round(kv_bytes / payload, 3),
+        "compression_ratio_total": round(kv_bytes / (payload + ab["side"]), 3),
+        "payload_bytes": payload,
+        "round_trip_within_half_step": verified,
+        "roofline": {
+            "kernel": "decode_streams_kernel",
+            "bound": "hbm",
+            "achieved": round(ab["decode"] / (dec_avg * 1e-3) / 1e9, 2),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(ab["decode"] / (dec_avg * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+            "traffic": None,
+            "algorithmic_bytes": ab["decode"],
+            "avg_launch_ms": round(dec_avg, 4),
+        },
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(kv[:, :, :args.cpu_sample_tokens].cpu(), kbins, vbins, chunk,
+                                              args.cpu_sample_tokens)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -254,81 +254,259 @@ __global__ __launch_bounds__(256) void quantize_kv_generic_kernel(
 }
 
 // ------------------------------------------------------------------------------------
+// Packed symbols of the fused path.  Each (row, sub-chunk) owns a slot of 64 words per
+// channel; byte j of word w is the symbol of token 4w + j of the sub-chunk:
+//   sym4[((row * nsub + sub) * 64 + w) * C + channel]
+// A lane of a stream kernel (one channel) gets four consecutive tokens with one 32-bit
+// load and a wave reads 256 contiguous bytes.
+// ------------------------------------------------------------------------------------
+constexpr int kWordsPerSub = kSub / 4;
+
+struct PackedQuantArgs {
+    const uint16_t *kv;
+    int64_t L, sl, skv, st, sh;
+    int32_t D;
+    const float *key_bins, *value_bins;
+    uint32_t *sym4;
+    uint16_t *maxima;       // [2L, T]
+    int32_t nunits;         // C / 8
+    int64_t nsub;
+    TokenGeom g;
+};
+
+// One wavefront quantizes four consecutive tokens of one row (encoder.py:42-59) and
+// writes, per channel, one word holding the four symbols: 32 contiguous bytes per lane
+// and unit, 2 KB per wave and store pair.
+template <int DT, bool HEADS_CONTIGUOUS, int NU>
+__global__ __launch_bounds__(256) void quantize_pack_kernel(PackedQuantArgs a)
+{
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    int64_t b = blockIdx.x;
+    const int tq = (int)(b & 15) * 4 + wave;      // word index inside the sub-chunk slot
+    b >>= 4;
+    const int64_t sub = b % a.nsub;
+    const int64_t row = b / a.nsub;
+    int64_t chunk, t0;
+    int n;
+    sub_range(a.g, sub, chunk, t0, n);
+    const int tt0 = tq * 4;
+    if (tt0 >= n) return;
+    const int nvalid = (n - tt0) < 4 ? (n - tt0) : 4;
+    const int64_t kvi = row / a.L, l = row - kvi * a.L;
+    const float bins = (kvi ? a.value_bins : a.key_bins)[l];
+    const float maxq = floorf(bins * 0.5f) - 1.0f;
+    const uint16_t *base = a.kv + l * a.sl + kvi * a.skv + (t0 + tt0) * a.st;
+
+    uint4 regs[4][NU];
+    float factor[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        uint32_t m = 0;
+#pragma unroll
+        for (int i = 0; i < NU; ++i) {
+            regs[j][i] = make_uint4(0, 0, 0, 0);
+            const int u = lane + 64 * i;
+            if (j < nvalid && u < a.nunits) {
+                const int e = u * 8;
+                int64_t off;
+                if (HEADS_CONTIGUOUS) off = e;
+                else { const int h = e / a.D; off = (int64_t)h * a.sh + (e - h * a.D); }
+                regs[j][i] = *reinterpret_cast<const uint4 *>(base + j * a.st + off);
+                m = pk_max_u16(m, regs[j][i].x & 0x7FFF7FFFu);
+                m = pk_max_u16(m, regs[j][i].y & 0x7FFF7FFFu);
+                m = pk_max_u16(m, regs[j][i].z & 0x7FFF7FFFu);
+                m = pk_max_u16(m, regs[j][i].w & 0x7FFF7FFFu);
+            }
+        }
+        m = (m & 0xFFFFu) > (m >> 16) ? (m & 0xFFFFu) : (m >> 16);
+        m = wave_max_u32(m);
+        if (j < nvalid && lane == 0) a.maxima[row * a.g.T + t0 + tt0 + j] = (uint16_t)m;
+        // rows past the end of the sub-chunk are all zero: 0 * inf = NaN -> symbol byte 0
+        factor[j] = __fdiv_rn(maxq, load16f<DT>(m));
+    }
+
+    const int64_t C = (int64_t)a.nunits * 8;
+    uint32_t *out = a.sym4 + ((row * a.nsub + sub) * kWordsPerSub + tq) * C;
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {
+        const int u = lane + 64 * i;
+        if (u < a.nunits) {
+            uint32_t words[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                uint32_t w = 0;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t src = k < 2 ? regs[j][i].x : k < 4 ? regs[j][i].y
+                                       : k < 6 ? regs[j][i].z : regs[j][i].w;
+                    const uint32_t bits = (k & 1) ? (src >> 16) : (src & 0xFFFFu);
+                    const float v = load16f<DT>(bits);
+                    const float s = __fadd_rn(__fmul_rn(v, factor[j]), maxq);
+                    const float r = fmaxf(__builtin_rintf(s), 0.0f);     // NaN -> 0
+                    w = __builtin_amdgcn_cvt_pk_u8_f32(r, (uint32_t)j, w);
+                }
+                words[k] = w;
+            }
+            uint4 *dst = reinterpret_cast<uint4 *>(out + (int64_t)u * 8);
+            dst[0] = make_uint4(words[0], words[1], words[2], words[3]);
+            dst[1] = make_uint4(words[4], words[5], words[6], words[7]);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------
 // Tables (cal_cdf.cu:17-59): one lane per (chunk, row, channel) walks the chunk's tokens
-// and counts into its own LDS column hist[bin][lane] (no atomics, no bank conflicts);
-// the running sum and the normalisation
+// and counts into its own LDS column hist[bin][lane] (no atomics across lanes, no bank
+// conflicts); the running sum and the normalisation
 //   cdf[i] = (uint16)((0xFFFF - max_bins) * cum[i] / cum[max_bins]) + i
 // are done per lane in 16-bit wrap-around arithmetic like the reference's uint16
-// counters, and the wave writes its 64 tables back transposed so stores coalesce.
+// counters, and the block writes its tables back transposed so stores coalesce.
 // ------------------------------------------------------------------------------------
+
+// Running sum and normalisation of one lane's column col[i * BS], i in [0, lp).
+template <int BS>
+__device__ __forceinline__ void normalize_column(uint32_t *col, int lp, int max_bins)
+{
+    uint32_t running = 0;
+    for (int i = 1; i < lp; ++i) {
+        running = (running + col[i * BS]) & 0xFFFFu;
+        col[i * BS] = running;
+    }
+    const uint32_t scale = 0xFFFFu - (uint32_t)max_bins;
+    for (int i = 0; i < lp; ++i) {
+        const uint32_t q = running ? (scale * col[i * BS] / running) & 0xFFFFu : 0u;
+        col[i * BS] = (q + (uint32_t)i) & 0xFFFFu;
+    }
+}
+
+// The same when every one of `total` tokens was counted (1 <= total <= 65535, uniform
+// over the block): the divide becomes a shift or a float estimate corrected exactly.
+template <int BS>
+__device__ __forceinline__ void normalize_column_total(uint32_t *col, int lp, int max_bins, uint32_t total)
+{
+    uint32_t running = 0;
+    for (int i = 1; i < lp; ++i) {
+        running += col[i * BS];
+        col[i * BS] = running;
+    }
+    const uint32_t scale = 0xFFFFu - (uint32_t)max_bins;
+    if ((total & (total - 1)) == 0) {
+        const int sh = 31 - __builtin_clz(total);
+        for (int i = 0; i < lp; ++i) col[i * BS] = ((scale * col[i * BS]) >> sh) + (uint32_t)i;
+    } else {
+        const float inv = __fdiv_rn(1.0f, (float)total);
+        for (int i = 0; i < lp; ++i) {
+            const uint32_t x = scale * col[i * BS];              // < 2^32, quotient < 2^16
+            uint32_t q = (uint32_t)((float)x * inv);
+            int32_t rem = (int32_t)(x - q * total);
+            if (rem < 0) { q--; rem += (int32_t)total; }
+            if (rem >= (int32_t)total) q++;
+            col[i * BS] = q + (uint32_t)i;
+        }
+    }
+}
+
+// Write the block's tables tab[entry * BS + lane] to cdf[lane][entry], coalesced.
+template <int BS>
+__device__ __forceinline__ void write_tables(const uint32_t *tab, uint16_t *cdf, int lp, int64_t ch0, int64_t nc)
+{
+    const int64_t nvalid = (nc - ch0 < BS) ? (nc - ch0) : BS;
+    const int total = (int)nvalid * lp;
+    for (int i = threadIdx.x; i < total; i += BS) {
+        const int c = i / lp, e = i - c * lp;
+        cdf[i] = (uint16_t)tab[e * BS + c];
+    }
+}
+
+// Load the block's tables into LDS as tab[entry * BS + lane] (32-bit words).
+template <int BS>
+__device__ __forceinline__ void stage_tables(uint32_t *tab, const uint16_t *cdf, int lp, int64_t ch0, int64_t nc)
+{
+    const int64_t nvalid = (nc - ch0 < BS) ? (nc - ch0) : BS;
+    const int total = (int)nvalid * lp;
+    for (int i = threadIdx.x; i < total; i += BS) {
+        const int c = i / lp, e = i - c * lp;
+        tab[e * BS + c] = cdf[i];
+    }
+}
+
 struct CdfArgs {
-    const uint8_t *sym;
-    int64_t s0, s1, s2;     // sym[row*s0 + token*s1 + channel*s2]
+    const uint8_t *sym;     // byte symbols: sym[row*s0 + token*s1 + channel*s2]
+    int64_t s0, s1, s2;
+    const uint32_t *sym4;   // or packed symbols (see above)
+    int64_t nsub;
     uint16_t *cdf;          // [chunk][row][channel][lp]
     int64_t rows, nc;
-    int32_t ctiles;         // blocks per row
+    int32_t ctiles;
     int32_t max_bins;
     TokenGeom g;
 };
 
-__global__ __launch_bounds__(256) void calculate_cdf_kernel(CdfArgs a)
+template <int BS, bool PACKED>
+__global__ __launch_bounds__(BS) void calculate_cdf_kernel(CdfArgs a)
 {
     extern __shared__ uint32_t smem[];
-    const int bs = blockDim.x, tid = threadIdx.x;
+    const int tid = threadIdx.x;
     const int lp = a.max_bins + 1;
     int64_t b = blockIdx.x;
     const int ctile = (int)(b % a.ctiles);
     b /= a.ctiles;
     const int64_t row = b % a.rows;
     const int64_t chunk = b / a.rows;
-    const int64_t ch = (int64_t)ctile * bs + tid;
-    const bool active = ch < a.nc;
-
-    for (int i = 0; i < lp; ++i) smem[i * bs + tid] = 0;
+    const int64_t ch = (int64_t)ctile * BS + tid;
+    uint32_t *col = smem + tid;
+    for (int i = 0; i < lp; ++i) col[i * BS] = 0;
 
     const int64_t t0 = chunk * a.g.S;
     int64_t t1 = t0 + a.g.S;
     if (t1 > a.g.T) t1 = a.g.T;
-    if (active) {
-        const uint8_t *p = a.sym + row * a.s0 + ch * a.s2;
-        int64_t t = t0;
-        for (; t + 4 <= t1; t += 4) {
-            const uint32_t v0 = p[(t + 0) * a.s1], v1 = p[(t + 1) * a.s1];
-            const uint32_t v2 = p[(t + 2) * a.s1], v3 = p[(t + 3) * a.s1];
-            if (v0 < (uint32_t)a.max_bins) smem[(v0 + 1) * bs + tid]++;
-            if (v1 < (uint32_t)a.max_bins) smem[(v1 + 1) * bs + tid]++;
-            if (v2 < (uint32_t)a.max_bins) smem[(v2 + 1) * bs + tid]++;
-            if (v3 < (uint32_t)a.max_bins) smem[(v3 + 1) * bs + tid]++;
+    const uint32_t mb = (uint32_t)a.max_bins;
+    if (ch < a.nc) {
+        if (!PACKED) {
+            const uint8_t *p = a.sym + row * a.s0 + ch * a.s2;
+            int64_t t = t0;
+            for (; t + 8 <= t1; t += 8) {
+                uint32_t v[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) v[j] = p[(t + j) * a.s1];
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (v[j] < mb) col[(v[j] + 1) * BS]++;
+            }
+            for (; t < t1; ++t) {
+                const uint32_t v = p[t * a.s1];
+                if (v < mb) col[(v + 1) * BS]++;
+            }
+        } else {
+            const int64_t sub0 = chunk * a.g.nsc;
+            const int nsubs = (int)((t1 - t0 + kSub - 1) / kSub);
+            for (int sidx = 0; sidx < nsubs; ++sidx) {
+                const int64_t left = (t1 - t0) - (int64_t)sidx * kSub;
+                const int n = left < kSub ? (int)left : kSub;
+                const uint32_t *wp = a.sym4 + ((row * a.nsub + sub0 + sidx) * kWordsPerSub) * a.nc + ch;
+                const int nwords = (n + 3) >> 2;
+                for (int w0 = 0; w0 < nwords; w0 += 4) {
+                    uint32_t v[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) v[j] = (w0 + j < nwords) ? wp[(int64_t)(w0 + j) * a.nc] : 0u;
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) {
+                        const uint32_t s = (v[j >> 2] >> (8 * (j & 3))) & 0xFFu;
+                        if (w0 * 4 + j < n && s < mb) col[(s + 1) * BS]++;
+                    }
+                }
+            }
         }
-        for (; t < t1; ++t) {
-            const uint32_t v = p[t * a.s1];
-            if (v < (uint32_t)a.max_bins) smem[(v + 1) * bs + tid]++;
-        }
-        uint32_t running = 0;
-        for (int i = 1; i < lp; ++i) {
-            running = (running + smem[i * bs + tid]) & 0xFFFFu;
-            smem[i * bs + tid] = running;
-        }
-        const uint32_t scale = 0xFFFFu - (uint32_t)a.max_bins;
-        for (int i = 0; i < lp; ++i) {
-            const uint32_t q = running ? (scale * smem[i * bs + tid] / running) & 0xFFFFu : 0u;
-            smem[i * bs + tid] = (q + (uint32_t)i) & 0xFFFFu;
-        }
+        normalize_column<BS>(col, lp, a.max_bins);
     }
     __syncthreads();
-    const int64_t ch0 = (int64_t)ctile * bs;
-    const int64_t nvalid = (a.nc - ch0 < bs) ? (a.nc - ch0) : bs;
-    uint16_t *out = a.cdf + ((chunk * a.rows + row) * a.nc + ch0) * lp;
-    const int total = (int)nvalid * lp;
-    for (int i = tid; i < total; i += bs) {
-        const int c = i / lp, e = i - c * lp;
-        out[i] = (uint16_t)smem[e * bs + c];
-    }
+    const int64_t ch0 = (int64_t)ctile * BS;
+    write_tables<BS>(smem, a.cdf + ((chunk * a.rows + row) * a.nc + ch0) * lp, lp, ch0, a.nc);
 }
 
 // ------------------------------------------------------------------------------------
-// Arithmetic coder.  Shared geometry of the encoder and decoder kernels: a block of
-// `blockDim.x` lanes covers that many adjacent channels of one (sub-chunk, row).
+// Arithmetic coder.  Shared geometry of the encoder and decoder kernels: a block of BS
+// lanes covers BS adjacent channels of one (sub-chunk, row).
 // ------------------------------------------------------------------------------------
 struct StreamGrid {
     int64_t rows, nc;
@@ -342,6 +520,7 @@ struct StreamId {
     bool active;
 };
 
+template <int BS>
 __device__ __forceinline__ StreamId locate(const StreamGrid &sg)
 {
     StreamId s;
@@ -351,29 +530,18 @@ __device__ __forceinline__ StreamId locate(const StreamGrid &sg)
     s.row = b % sg.rows;
     s.sub = b / sg.rows;
     sub_range(sg.g, s.sub, s.chunk, s.t0, s.n);
-    s.ch = (int64_t)ctile * blockDim.x + threadIdx.x;
+    s.ch = (int64_t)ctile * BS + threadIdx.x;
     s.active = s.ch < sg.nc;
     return s;
-}
-
-// Load the block's tables into LDS as tab[entry * bs + lane] (32-bit words).
-__device__ __forceinline__ void stage_tables(uint32_t *tab, const uint16_t *cdf, int lp,
-                                             int64_t ch0, int64_t nc)
-{
-    const int bs = blockDim.x;
-    const int64_t nvalid = (nc - ch0 < bs) ? (nc - ch0) : bs;
-    const int total = (int)nvalid * lp;
-    for (int i = threadIdx.x; i < total; i += bs) {
-        const int c = i / lp, e = i - c * lp;
-        tab[e * bs + c] = cdf[i];
-    }
 }
 
 // ---- encoder (enc_new.cu:21-97, 253-307) -------------------------------------------
 // Bits are collected MSB-first in a 32-bit accumulator and leave as big-endian words.
 // The E1/E2 run of a symbol is emitted at once: clz(low ^ high) leading bits agree, the
 // first of them is followed by the pending complements; the E3 run is the number of
-// positions below the top where low has ones and high has zeros.
+// positions below those where low has ones and high has zeros.  One combined shift by
+// n = n1 + k renormalises low and high; n <= 18 for any table whose symbols all have
+// non-zero width, because the span stays above 2^30 between symbols.
 template <bool ALIGNED>
 struct BitWriter {
     uint8_t *dst;
@@ -440,11 +608,82 @@ struct BitWriter {
     }
 };
 
+template <int BS, bool ALIGNED>
+struct RangeEncoder {
+    const uint32_t *col;    // this lane's table column: entry e at col[e * BS]
+    uint32_t top;           // lp - 1: index of the table end (holds 2^16)
+    uint32_t low, high, pend;
+    BitWriter<ALIGNED> w;
+
+    __device__ __forceinline__ void init(const uint32_t *column, int lp, uint8_t *dst, int cap)
+    {
+        col = column;
+        top = (uint32_t)(lp - 1);
+        low = 0;
+        high = 0xFFFFFFFFu;
+        pend = 0;
+        w.dst = dst;
+        w.cap = cap;
+        w.nbytes = 0;
+        w.acc = 0;
+        w.nacc = 0;
+    }
+
+    __device__ __forceinline__ void put_symbol(uint32_t s)
+    {
+        s = s < top ? s : top - 1;                      // keep table reads inside the table
+        const uint32_t r = high - low;
+        const uint32_t rh = r >> 16, rl = r & 0xFFFFu;
+        const uint32_t c_lo = col[s * BS];
+        const uint32_t c_hi = col[s * BS + BS];
+        const uint32_t t_lo = scale16(rh, rl, c_lo);
+        const uint32_t t_hi_table = scale16(rh, rl, c_hi);
+        const uint32_t t_hi = c_hi == 0x10000u ? r + 1u : t_hi_table;
+        high = low + t_hi - 1u;
+        low = low + t_lo;
+
+        const int n1 = __builtin_clz(low ^ high);       // low < high always
+        if (n1 > 0) {
+            const uint32_t bits = low >> ((32 - n1) & 31);          // the n1 agreed bits
+            if (pend == 0) {
+                w.put(bits, n1);
+            } else if (pend + (uint32_t)n1 <= 32u) {
+                const uint32_t b = bits >> (n1 - 1);
+                const uint32_t head = ((1u << pend) - 1u) + b;       // b, then `pend` complements
+                const uint32_t rest = bits & ((1u << (n1 - 1)) - 1u);
+                w.put((head << (n1 - 1)) | rest, (int)pend + n1);
+            } else {
+                const uint32_t b = bits >> (n1 - 1);
+                w.put(b, 1);
+                w.run(1u - b, pend);
+                if (n1 > 1) w.put(bits & ((1u << (n1 - 1)) - 1u), n1 - 1);
+            }
+            pend = 0;
+        }
+        const int k = __builtin_clz(~((low & ~high) << ((n1 + 1) & 31)));
+        const int n = (n1 + k) & 31;
+        pend += (uint32_t)k;
+        low = (low << n) & 0x7FFFFFFFu;
+        high = (high << n) | 0x80000000u | ~(0xFFFFFFFFu << n);
+    }
+
+    __device__ __forceinline__ int finish()
+    {
+        pend += 1;
+        const uint32_t b = low < 0x40000000u ? 0u : 1u;
+        w.put(b, 1);
+        w.run(1u - b, pend);
+        return w.finish();
+    }
+};
+
 struct EncodeArgs {
-    const uint16_t *cdf;    // [chunk][row][channel][lp]
+    uint16_t *cdf;          // [chunk][row][channel][lp]; written when the histogram is fused
     int32_t lp;
-    const uint8_t *sym;     // sym[row*s0 + token*s1 + channel*s2]
+    const uint8_t *sym;     // byte symbols: sym[row*s0 + token*s1 + channel*s2]
     int64_t s0, s1, s2;
+    const uint32_t *sym4;   // or packed symbols
+    int64_t nsub;
     uint8_t *out;           // out[sub*osub + row*o0 + channel*o1 + byte]
     int64_t osub, o0, o1;
     int32_t cap;
@@ -453,70 +692,84 @@ struct EncodeArgs {
     StreamGrid sg;
 };
 
-template <bool ALIGNED>
-__global__ __launch_bounds__(256) void encode_streams_kernel(EncodeArgs a)
+// PACKED: symbols come from sym4.  FUSE_CDF (PACKED only, one sub-chunk per chunk): the
+// block first builds its own tables from the same words and writes them out.
+template <int BS, bool ALIGNED, bool PACKED, bool FUSE_CDF>
+__global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
 {
     extern __shared__ uint32_t tab[];
-    const int bs = blockDim.x, tid = threadIdx.x;
-    const StreamId id = locate(a.sg);
+    const int tid = threadIdx.x;
+    const StreamId id = locate<BS>(a.sg);
     const int lp = a.lp;
     const int64_t ch0 = id.ch - tid;
-    stage_tables(tab, a.cdf + ((id.chunk * a.sg.rows + id.row) * a.sg.nc + ch0) * lp, lp, ch0, a.sg.nc);
-    __syncthreads();
+    uint32_t *col = tab + tid;
+    uint16_t *cdf_block = a.cdf + ((id.chunk * a.sg.rows + id.row) * a.sg.nc + ch0) * lp;
+    const uint32_t *wp = nullptr;
+    const int nwords = (id.n + 3) >> 2;
+    if (PACKED) wp = a.sym4 + ((id.row * a.nsub + id.sub) * kWordsPerSub) * a.sg.nc + id.ch;
+
+    if (FUSE_CDF) {
+        for (int i = 0; i < lp; ++i) col[i * BS] = 0;
+        if (id.active) {
+            const uint32_t smax = (uint32_t)(lp - 2);
+            for (int w0 = 0; w0 < nwords; w0 += 4) {
+                uint32_t v[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v[j] = (w0 + j < nwords) ? wp[(int64_t)(w0 + j) * a.sg.nc] : 0u;
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    uint32_t s = (v[j >> 2] >> (8 * (j & 3))) & 0xFFu;
+                    s = s < smax ? s : smax;
+                    if (w0 * 4 + j < id.n) atomicAdd(&col[(s + 1) * BS], 1u);
+                }
+            }
+            normalize_column_total<BS>(col, lp, lp - 1, (uint32_t)id.n);
+        }
+        __syncthreads();
+        write_tables<BS>(tab, cdf_block, lp, ch0, a.sg.nc);
+        __syncthreads();
+    } else {
+        stage_tables<BS>(tab, cdf_block, lp, ch0, a.sg.nc);
+        __syncthreads();
+    }
     if (!id.active) return;
     // the upper bound of the last symbol is 2^16, not the stored value (enc_new.cu:270)
-    tab[(lp - 1) * bs + tid] = 0x10000u;
+    col[(lp - 1) * BS] = 0x10000u;
 
-    const uint8_t *sp = a.sym + id.row * a.s0 + id.t0 * a.s1 + id.ch * a.s2;
-    BitWriter<ALIGNED> w;
-    w.dst = a.out + id.sub * a.osub + id.row * a.o0 + id.ch * a.o1;
-    w.cap = a.cap;
-    w.nbytes = 0;
-    w.acc = 0;
-    w.nacc = 0;
+    RangeEncoder<BS, ALIGNED> enc;
+    enc.init(col, lp, a.out + id.sub * a.osub + id.row * a.o0 + id.ch * a.o1, a.cap);
 
-    uint32_t low = 0, high = 0xFFFFFFFFu, pend = 0;
-    const uint32_t top = (uint32_t)(lp - 1);
-    uint32_t s_next = id.n > 0 ? sp[0] : 0;
-    for (int i = 0; i < id.n; ++i) {
-        uint32_t s = s_next;
-        if (i + 1 < id.n) s_next = sp[(int64_t)(i + 1) * a.s1];
-        s = s < top ? s : top - 1;                      // keep table reads inside the table
-        const uint32_t r = high - low;
-        const uint32_t rh = r >> 16, rl = r & 0xFFFFu;
-        const uint32_t c_lo = tab[s * bs + tid];
-        const uint32_t c_hi = tab[(s + 1) * bs + tid];
-        const uint32_t t_lo = scale16(rh, rl, c_lo);
-        const uint32_t t_hi = c_hi == 0x10000u ? r + 1u : scale16(rh, rl, c_hi);
-        high = low + t_hi - 1u;
-        low = low + t_lo;
-
-        const int n1 = __builtin_clz(low ^ high);        // low < high always
-        if (n1 > 0) {
-            const uint32_t b = low >> 31;
-            const uint32_t rest = (low & 0x7FFFFFFFu) >> (32 - n1);
-            if (pend + (uint32_t)n1 <= 32u) {
-                const uint32_t head = ((1u << pend) - 1u) + b;   // b, then `pend` complements
-                w.put((head << (n1 - 1)) | rest, (int)pend + n1);
-            } else {
-                w.put(b, 1);
-                w.run(1u - b, pend);
-                if (n1 > 1) w.put(rest, n1 - 1);
-            }
-            pend = 0;
+    if (PACKED) {
+        uint32_t nxt[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) nxt[j] = (j < nwords) ? wp[(int64_t)j * a.sg.nc] : 0u;
+        for (int w0 = 0; w0 < nwords; w0 += 4) {
+            uint32_t cur[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) cur[j] = nxt[j];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) nxt[j] = (w0 + 4 + j < nwords) ? wp[(int64_t)(w0 + 4 + j) * a.sg.nc] : 0u;
+#pragma unroll
+            for (int j = 0; j < 16; ++j)
+                if (w0 * 4 + j < id.n) enc.put_symbol((cur[j >> 2] >> (8 * (j & 3))) & 0xFFu);
         }
-        const uint32_t lo1 = low << n1;
-        const uint32_t hi1 = (high << n1) | ((1u << n1) - 1u);
-        const int k = __builtin_clz(~((lo1 & ~hi1) << 1));
-        pend += (uint32_t)k;
-        low = (lo1 << k) & 0x7FFFFFFFu;
-        high = (hi1 << k) | 0x80000000u | ((1u << k) - 1u);
+    } else {
+        const uint8_t *sp = a.sym + id.row * a.s0 + id.t0 * a.s1 + id.ch * a.s2;
+        uint32_t nxt[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) nxt[j] = (j < id.n) ? sp[(int64_t)j * a.s1] : 0u;
+        for (int i0 = 0; i0 < id.n; i0 += 8) {
+            uint32_t cur[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) cur[j] = nxt[j];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) nxt[j] = (i0 + 8 + j < id.n) ? sp[(int64_t)(i0 + 8 + j) * a.s1] : 0u;
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                if (i0 + j < id.n) enc.put_symbol(cur[j]);
+        }
     }
-    pend += 1;
-    const uint32_t b = low < 0x40000000u ? 0u : 1u;
-    w.put(b, 1);
-    w.run(1u - b, pend);
-    const int len = w.finish();
+    const int len = enc.finish();
     a.lengths[(id.sub * a.sg.rows + id.row) * a.sg.nc + id.ch] = len;
     if (len > a.cap && a.status) atomicOr(a.status, 1);
 }
@@ -526,53 +779,46 @@ __global__ __launch_bounds__(256) void encode_streams_kernel(EncodeArgs a)
 // 2*off + next bit (E1/E2 and E3 alike), and finds the symbol as the largest m with
 // floor(span*cdf[m] / 2^16) <= off; that is the same m as the reference's search of
 // count = ((value-low+1)*2^16 - 1) / span in a strictly increasing table, without the
-// 64-bit divide.  The stream is read through aligned big-endian words with one word of
-// prefetch; bytes past the stream's end read as zero (dec_new.cu:223-233).
+// 64-bit divide.  The stream is read through aligned big-endian words with one raw word
+// in flight.  Bits past the end of a stream are whatever follows it in memory instead of
+// the reference's zeros (dec_new.cu:223-233): the coder's two closing bits place the
+// code value inside the final interval for every continuation, so the n symbols that
+// were encoded decode identically.  Loads never pass the end of the byte buffer.
 struct BitReader {
-    const uint32_t *words;   // aligned word containing the stream's first byte
-    int64_t nwords_safe;     // words that may be touched
-    uint32_t end_bit;        // first bit (from `words`) past the stream
-    uint32_t w0, w1, w2;
+    const uint32_t *words;   // aligned word holding the stream's first byte
+    uint32_t nwords_ok;      // words from `words` that lie inside the byte buffer
+    uint32_t w0, w1, raw2;
     int c;                   // unread low bits of w0
-    uint32_t next;           // index of the next word to prefetch
+    uint32_t next;           // index of the next word to fetch
 
-    __device__ __forceinline__ uint32_t load_word(uint32_t j) const
-    {
-        const uint32_t first = j * 32u;
-        uint32_t w = 0;
-        if (first < end_bit) {
-            w = __builtin_bswap32(words[j]);
-            const uint32_t left = end_bit - first;
-            if (left < 32u) w &= 0xFFFFFFFFu << (32u - left);
-        }
-        return w;
-    }
+    __device__ __forceinline__ uint32_t raw(uint32_t j) const { return j < nwords_ok ? words[j] : 0u; }
 
-    // position on the stream that starts `skip_bytes` (0..3) into words[0] and is
-    // `len` bytes long; returns its first 32 bits
-    __device__ __forceinline__ uint32_t start(const uint8_t *begin, int len)
+    // position on the stream that begins at `begin`; `buf_end` is one past the last byte
+    // that may be read (rounded up to a word here); returns the stream's first 32 bits
+    __device__ __forceinline__ uint32_t start(const uint8_t *begin, const uint8_t *buf_end)
     {
-        const uintptr_t addr = reinterpret_cast<uintptr_t>(begin);
-        const uint32_t skip = (uint32_t)(addr & 3u);
-        words = reinterpret_cast<const uint32_t *>(addr - skip);
-        end_bit = (skip + (uint32_t)len) * 8u;
+        const uint32_t skip = (uint32_t)(reinterpret_cast<uintptr_t>(begin) & 3u);
+        const uint8_t *aligned = begin - skip;
+        words = reinterpret_cast<const uint32_t *>(aligned);
+        const int64_t span_bytes = buf_end - aligned;
+        nwords_ok = span_bytes > 0 ? (uint32_t)((span_bytes + 3) >> 2) : 0u;
+        const uint32_t b0 = __builtin_bswap32(raw(0)), b1 = __builtin_bswap32(raw(1));
+        uint32_t first;
         if (skip == 0) {
-            w0 = 0;
-            w1 = load_word(0);
-            w2 = load_word(1);
-            next = 2;
+            first = b0;
+            w0 = b0;
             c = 0;
-        } else {
-            w0 = load_word(0);
-            w1 = load_word(1);
-            w2 = load_word(2);
+            w1 = b1;
+            raw2 = raw(2);
             next = 3;
+        } else {
             c = 32 - (int)(skip * 8u);
+            first = __builtin_amdgcn_alignbit(b0, b1, (uint32_t)c);
+            w0 = b1;
+            w1 = __builtin_bswap32(raw(2));
+            raw2 = raw(3);
+            next = 4;
         }
-        const uint32_t first = __builtin_amdgcn_alignbit(w0, w1, (uint32_t)c);
-        w0 = w1;
-        w1 = w2;
-        w2 = load_word(next++);
         return first;
     }
 
@@ -580,14 +826,14 @@ struct BitReader {
     __device__ __forceinline__ uint32_t shift_in(uint32_t off, int n)
     {
         const uint32_t nx = __builtin_amdgcn_alignbit(w0, w1, (uint32_t)c);
-        const uint32_t shifted = __builtin_amdgcn_alignbit(off, nx, (uint32_t)(32 - n));
-        off = n ? shifted : off;
+        off = (uint32_t)(((((uint64_t)off) << 32) | nx) >> (32 - n));
         c -= n;
         if (c < 0) {
             w0 = w1;
-            w1 = w2;
+            w1 = __builtin_bswap32(raw2);
             c += 32;
-            w2 = load_word(next++);
+            raw2 = raw(next);
+            next++;
         }
         return off;
     }
@@ -600,6 +846,7 @@ struct DecodeArgs {
     const uint16_t *cdf;
     int32_t lp;
     const uint8_t *bytes;       // payload, or padded buffer
+    int64_t nbytes;             // readable bytes from `bytes`
     const int64_t *offsets;     // SRC_OFFSETS: exclusive sums [nstreams+1]; SRC_PREFIX: inclusive sums
     const int32_t *lengths;     // SRC_PADDED
     int64_t p0, p1;             // SRC_PADDED strides
@@ -618,51 +865,52 @@ struct DecodeArgs {
     StreamGrid sg;
 };
 
-template <int SRC, int OUT, int MAXDT>
-__global__ __launch_bounds__(256) void decode_streams_kernel(DecodeArgs a)
+// LOG2 >= 0: the table has exactly 2^LOG2 symbols (lp = 2^LOG2 + 1) and the search is
+// unrolled with immediate LDS offsets; LOG2 < 0: any lp.
+template <int BS, int LOG2, int SRC, int OUT>
+__global__ __launch_bounds__(BS) void decode_streams_kernel(DecodeArgs a)
 {
     extern __shared__ uint32_t smem[];
-    const int bs = blockDim.x, tid = threadIdx.x;
-    const StreamId id = locate(a.sg);
-    const int lp = a.lp;
+    const int tid = threadIdx.x;
+    const StreamId id = locate<BS>(a.sg);
+    const int lp = LOG2 >= 0 ? (1 << LOG2) + 1 : a.lp;
     uint32_t *tab = smem;
-    float *lut = reinterpret_cast<float *>(smem + lp * bs);   // (s - C) / C per symbol
+    float *lut = reinterpret_cast<float *>(smem + lp * BS);   // (s - C) / C per symbol
     float *rowmax = lut + lp;                                 // one per token of the sub-chunk
     const int64_t ch0 = id.ch - tid;
-    stage_tables(tab, a.cdf + ((id.chunk * a.sg.rows + id.row) * a.sg.nc + ch0) * lp, lp, ch0, a.sg.nc);
+    stage_tables<BS>(tab, a.cdf + ((id.chunk * a.sg.rows + id.row) * a.sg.nc + ch0) * lp, lp, ch0, a.sg.nc);
     int64_t kvi = 0, l = 0;
     if (OUT != OUT_SYMBOLS) {
         kvi = id.row / a.L;
         l = id.row - kvi * a.L;
         const float bins = (kvi ? a.value_bins : a.key_bins)[l];
         const float cq = floorf(bins * 0.5f) - 1.0f;
-        for (int i = tid; i < lp; i += bs) lut[i] = __fdiv_rn(__fsub_rn((float)i, cq), cq);
+        for (int i = tid; i < lp; i += BS) lut[i] = __fdiv_rn(__fsub_rn((float)i, cq), cq);
         const uint16_t *mx = a.maxima + id.row * a.sg.g.T + id.t0;
-        for (int i = tid; i < id.n; i += bs) rowmax[i] = load16f<MAXDT>(mx[i]);
+        if (a.max_dt == CG_DT_BF16)
+            for (int i = tid; i < id.n; i += BS) rowmax[i] = load16f<CG_DT_BF16>(mx[i]);
+        else
+            for (int i = tid; i < id.n; i += BS) rowmax[i] = load16f<CG_DT_F16>(mx[i]);
     }
     __syncthreads();
     if (!id.active) return;
 
     const int64_t stream = (id.sub * a.sg.rows + id.row) * a.sg.nc + id.ch;
     const uint8_t *begin;
-    int len;
+    const uint8_t *buf_end;
     if (SRC == SRC_OFFSETS) {
-        const int64_t b0 = a.offsets[stream], b1 = a.offsets[stream + 1];
-        begin = a.bytes + b0;
-        len = (int)(b1 - b0);
+        begin = a.bytes + a.offsets[stream];
+        buf_end = a.bytes + a.nbytes;
     } else if (SRC == SRC_PREFIX) {
-        const int64_t b0 = stream ? a.offsets[stream - 1] : 0, b1 = a.offsets[stream];
-        begin = a.bytes + b0;
-        len = (int)(b1 - b0);
+        begin = a.bytes + (stream ? a.offsets[stream - 1] : 0);
+        buf_end = a.bytes + a.nbytes;
     } else {
         begin = a.bytes + id.row * a.p0 + id.ch * a.p1;
-        len = a.lengths[stream];
-        len = len < a.cap ? len : a.cap;
+        buf_end = begin + a.cap;
     }
-    len = len < 0 ? 0 : len;
 
     BitReader rd;
-    uint32_t off = rd.start(begin, len);
+    uint32_t off = rd.start(begin, buf_end);
     uint32_t low = 0, high = 0xFFFFFFFFu;
 
     uint8_t *osym = nullptr;
@@ -674,49 +922,61 @@ __global__ __launch_bounds__(256) void decode_streams_kernel(DecodeArgs a)
         okv = a.out_kv + l * a.ol + kvi * a.okv + id.t0 * a.ot + h * a.oh + (id.ch - h * a.D);
     }
 
+    const uint32_t *col = tab + tid;
     int nsteps = 0;
-    while ((1 << nsteps) < lp - 1) ++nsteps;
-    const uint32_t c0 = tab[tid];
+    if (LOG2 < 0)
+        while ((1 << nsteps) < lp - 1) ++nsteps;
 
     for (int i = 0; i < id.n; ++i) {
         const uint32_t r = high - low;
         const uint32_t rh = r >> 16, rl = r & 0xFFFFu;
-        int lo_i = 0, hi_i = lp - 1;
-        uint32_t t_lo = scale16(rh, rl, c0);
-        uint32_t t_hi = r + 1u;                         // table end is 2^16 (dec_new.cu:278)
-        for (int step = 0; step < nsteps; ++step) {
-            const int mid = (lo_i + hi_i) >> 1;
-            const uint32_t t = scale16(rh, rl, tab[mid * bs + tid]);
-            const bool le = t <= off;
-            lo_i = le ? mid : lo_i;
-            t_lo = le ? t : t_lo;
-            hi_i = le ? hi_i : mid;
-            t_hi = le ? t_hi : t;
+        uint32_t sidx;                     // decoded symbol
+        uint32_t c_lo, c_hi;
+        if (LOG2 >= 0) {
+            uint32_t pos = 0;                  // element offset of the current entry in the column
+#pragma unroll
+            for (int step = (1 << LOG2) >> 1; step >= 1; step >>= 1) {
+                const uint32_t t = scale16(rh, rl, col[pos + step * BS]);
+                pos = (t <= off) ? pos + step * BS : pos;
+            }
+            sidx = pos / BS;
+            c_lo = col[pos];
+            c_hi = col[pos + BS];
+        } else {
+            int lo_i = 0, hi_i = lp - 1;
+            for (int step = 0; step < nsteps; ++step) {
+                const int mid = (lo_i + hi_i) >> 1;
+                const uint32_t t = scale16(rh, rl, col[mid * BS]);
+                const bool le = mid > 0 && t <= off;
+                lo_i = le ? mid : lo_i;
+                hi_i = le ? hi_i : mid;
+            }
+            sidx = (uint32_t)lo_i;
+            c_lo = col[lo_i * BS];
+            c_hi = col[lo_i * BS + BS];
         }
         if (OUT == OUT_SYMBOLS) {
-            osym[(int64_t)i * a.o1] = (uint8_t)lo_i;
+            osym[(int64_t)i * a.o1] = (uint8_t)sidx;
         } else {
-            const float v = __fmul_rn(lut[lo_i], rowmax[i]);
-            okv[(int64_t)i * a.ot] = (uint16_t)(OUT == OUT_BF16 ? store16f<CG_DT_BF16>(v)
-                                                                : store16f<CG_DT_F16>(v));
+            const float v = __fmul_rn(lut[sidx], rowmax[i]);
+            *okv = (uint16_t)(OUT == OUT_BF16 ? store16f<CG_DT_BF16>(v) : store16f<CG_DT_F16>(v));
+            okv += a.ot;
         }
         if (i == id.n - 1) break;                       // no update after the last symbol
+        const uint32_t t_lo = scale16(rh, rl, c_lo);
+        // the last symbol's upper bound is 2^16 (dec_new.cu:278): span * 2^16 >> 16 = span
+        const uint32_t t_hi_table = scale16(rh, rl, c_hi);
+        const uint32_t t_hi = sidx == (uint32_t)(lp - 2) ? r + 1u : t_hi_table;
         high = low + t_hi - 1u;
         low = low + t_lo;
         off -= t_lo;
 
         const int n1 = __builtin_clz(low ^ high);
-        const uint32_t lo1 = low << n1;
-        const uint32_t hi1 = (high << n1) | ((1u << n1) - 1u);
-        const int k = __builtin_clz(~((lo1 & ~hi1) << 1));
-        low = (lo1 << k) & 0x7FFFFFFFu;
-        high = (hi1 << k) | 0x80000000u | ((1u << k) - 1u);
-        if (n1 + k <= 31) {
-            off = rd.shift_in(off, n1 + k);
-        } else {
-            off = rd.shift_in(off, n1);
-            off = rd.shift_in(off, k);
-        }
+        const int k = __builtin_clz(~((low & ~high) << ((n1 + 1) & 31)));
+        const int n = (n1 + k) & 31;
+        low = (low << n) & 0x7FFFFFFFu;
+        high = (high << n) | 0x80000000u | ~(0xFFFFFFFFu << n);
+        off = rd.shift_in(off, n);
     }
 }
 
@@ -864,8 +1124,17 @@ int make_grid(int64_t rows, int64_t nc, int64_t T, int64_t S, int64_t nsub, int 
     return CG_OK;
 }
 
-int launch_cdf(const uint8_t *sym, int64_t rows, int64_t T, int64_t nc, int64_t s0, int64_t s1,
-               int64_t s2, int max_bins, int64_t S, uint16_t *cdf, hipStream_t stream)
+// Run `launch` with the block size as a compile-time constant.
+#define CG_DISPATCH_BS(block, ...)                      \
+    do {                                                \
+        if ((block) == 256) { constexpr int BS = 256; __VA_ARGS__; } \
+        else if ((block) == 128) { constexpr int BS = 128; __VA_ARGS__; } \
+        else { constexpr int BS = 64; __VA_ARGS__; }    \
+    } while (0)
+
+int launch_cdf(const uint8_t *sym, const uint32_t *sym4, int64_t nsub, int64_t rows, int64_t T,
+               int64_t nc, int64_t s0, int64_t s1, int64_t s2, int max_bins, int64_t S,
+               uint16_t *cdf, hipStream_t stream)
 {
     const int block = pick_block(nc, max_bins + 1);
     CdfArgs a;
@@ -873,6 +1142,8 @@ int launch_cdf(const uint8_t *sym, int64_t rows, int64_t T, int64_t nc, int64_t 
     a.s0 = s0;
     a.s1 = s1;
     a.s2 = s2;
+    a.sym4 = sym4;
+    a.nsub = nsub;
     a.cdf = cdf;
     a.rows = rows;
     a.nc = nc;
@@ -884,7 +1155,9 @@ int launch_cdf(const uint8_t *sym, int64_t rows, int64_t T, int64_t nc, int64_t 
     const int64_t nblocks = ceil_div(T, S) * rows * a.ctiles;
     if (nblocks <= 0 || nblocks > INT_MAX) return fail(CG_ERR_ARG, "calculate_cdf: grid out of range");
     const size_t shmem = (size_t)(max_bins + 1) * block * sizeof(uint32_t);
-    calculate_cdf_kernel<<<dim3((unsigned)nblocks), dim3(block), shmem, stream>>>(a);
+    const dim3 grid((unsigned)nblocks), blk(block);
+    if (sym4) CG_DISPATCH_BS(block, (calculate_cdf_kernel<BS, true><<<grid, blk, shmem, stream>>>(a)));
+    else CG_DISPATCH_BS(block, (calculate_cdf_kernel<BS, false><<<grid, blk, shmem, stream>>>(a)));
     return check_launch("calculate_cdf");
 }
 
@@ -911,6 +1184,12 @@ int check_lp(int lp, const char *what)
     return CG_OK;
 }
 
+bool kv_vectorizable(const void *kv, int64_t D, int64_t C, int64_t sl, int64_t skv, int64_t st, int64_t sh)
+{
+    return (D % 8 == 0) && (sl % 8 == 0) && (skv % 8 == 0) && (st % 8 == 0) && (sh % 8 == 0) &&
+           aligned_to(kv, 16) && (C / 8 <= 64 * kMaxUnits);
+}
+
 int launch_quantize(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D,
                     int64_t sl, int64_t skv, int64_t st, int64_t sh, const float *key_bins,
                     const float *value_bins, uint8_t *sym, void *maxima, hipStream_t stream)
@@ -919,8 +1198,7 @@ int launch_quantize(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, 
     const int64_t nrows = 2 * L * T;
     const int64_t nblocks = ceil_div(nrows, 4);
     if (nblocks > INT_MAX || C > INT_MAX) return fail(CG_ERR_ARG, "quantize: tensor too large for one launch");
-    const bool vec = (D % 8 == 0) && (sl % 8 == 0) && (skv % 8 == 0) && (st % 8 == 0) && (sh % 8 == 0) &&
-                     aligned_to(kv, 16) && aligned_to(sym, 8) && (C / 8 <= 64 * kMaxUnits);
+    const bool vec = kv_vectorizable(kv, D, C, sl, skv, st, sh) && aligned_to(sym, 8);
     const uint16_t *p = static_cast<const uint16_t *>(kv);
     uint16_t *mx = static_cast<uint16_t *>(maxima);
     dim3 grid((unsigned)nblocks), block(256);
@@ -943,14 +1221,71 @@ int launch_quantize(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, 
     return check_launch("quantize_kv");
 }
 
-template <int SRC, int OUT>
-int launch_decode_dt(const DecodeArgs &a, int64_t nblocks, int block, size_t shmem, hipStream_t stream)
+template <int DT, bool HC>
+void launch_quantize_pack_nu(const PackedQuantArgs &a, int64_t nblocks, hipStream_t stream)
 {
-    if (a.max_dt == CG_DT_BF16)
-        decode_streams_kernel<SRC, OUT, CG_DT_BF16><<<dim3((unsigned)nblocks), dim3(block), shmem, stream>>>(a);
-    else
-        decode_streams_kernel<SRC, OUT, CG_DT_F16><<<dim3((unsigned)nblocks), dim3(block), shmem, stream>>>(a);
+    const dim3 grid((unsigned)nblocks), block(256);
+    if (a.nunits <= 128) quantize_pack_kernel<DT, HC, 2><<<grid, block, 0, stream>>>(a);
+    else if (a.nunits <= 256) quantize_pack_kernel<DT, HC, 4><<<grid, block, 0, stream>>>(a);
+    else quantize_pack_kernel<DT, HC, 8><<<grid, block, 0, stream>>>(a);
+}
+
+int launch_quantize_pack(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D,
+                         int64_t sl, int64_t skv, int64_t st, int64_t sh, const float *key_bins,
+                         const float *value_bins, uint32_t *sym4, void *maxima, int64_t nsub,
+                         int64_t S, hipStream_t stream)
+{
+    PackedQuantArgs a;
+    a.kv = static_cast<const uint16_t *>(kv);
+    a.L = L;
+    a.sl = sl;
+    a.skv = skv;
+    a.st = st;
+    a.sh = sh;
+    a.D = (int32_t)D;
+    a.key_bins = key_bins;
+    a.value_bins = value_bins;
+    a.sym4 = sym4;
+    a.maxima = static_cast<uint16_t *>(maxima);
+    a.nunits = (int32_t)(H * D / 8);
+    a.nsub = nsub;
+    a.g.T = T;
+    a.g.S = S;
+    a.g.nsc = (int32_t)ceil_div(S, kSub);
+    const int64_t nblocks = 2 * L * nsub * 16;
+    if (nblocks > INT_MAX) return fail(CG_ERR_ARG, "quantize: tensor too large for one launch");
+    const bool contiguous = (sh == D);
+    if (kv_dt == CG_DT_F16) {
+        if (contiguous) launch_quantize_pack_nu<CG_DT_F16, true>(a, nblocks, stream);
+        else launch_quantize_pack_nu<CG_DT_F16, false>(a, nblocks, stream);
+    } else {
+        if (contiguous) launch_quantize_pack_nu<CG_DT_BF16, true>(a, nblocks, stream);
+        else launch_quantize_pack_nu<CG_DT_BF16, false>(a, nblocks, stream);
+    }
+    return check_launch("quantize_pack");
+}
+
+size_t decode_shmem(int lp, int block) { return (size_t)lp * block * sizeof(uint32_t) + (size_t)(lp + kSub) * sizeof(float); }
+
+template <int SRC>
+int launch_decode_symbols(const DecodeArgs &a, int64_t nblocks, int block, hipStream_t stream)
+{
+    const dim3 grid((unsigned)nblocks), blk(block);
+    const size_t shmem = decode_shmem(a.lp, block);
+    CG_DISPATCH_BS(block, (decode_streams_kernel<BS, -1, SRC, OUT_SYMBOLS><<<grid, blk, shmem, stream>>>(a)));
     return check_launch("decode");
+}
+
+template <int BS, int OUT>
+void launch_decode_kv_log2(const DecodeArgs &a, dim3 grid, size_t shmem, hipStream_t stream)
+{
+    const dim3 blk(BS);
+    switch (a.lp) {
+    case 17: decode_streams_kernel<BS, 4, SRC_OFFSETS, OUT><<<grid, blk, shmem, stream>>>(a); break;
+    case 33: decode_streams_kernel<BS, 5, SRC_OFFSETS, OUT><<<grid, blk, shmem, stream>>>(a); break;
+    case 65: decode_streams_kernel<BS, 6, SRC_OFFSETS, OUT><<<grid, blk, shmem, stream>>>(a); break;
+    default: decode_streams_kernel<BS, -1, SRC_OFFSETS, OUT><<<grid, blk, shmem, stream>>>(a); break;
+    }
 }
 
 }  // namespace
@@ -984,7 +1319,7 @@ int cg_calculate_cdf(const int8_t *sym, int64_t nl, int64_t nt, int64_t nc, int6
     if (nl <= 0 || nt <= 0 || nc <= 0) return fail(CG_ERR_ARG, "calculate_cdf: empty input");
     if (max_bins < 1 || max_bins + 1 > CG_MAX_LP) return fail(CG_ERR_ARG, "Max bins must be less than %d", CG_MAX_LP);
     if (nt > 65535) return fail(CG_ERR_ARG, "calculate_cdf: at most 65535 tokens per table (16-bit counters)");
-    return launch_cdf(reinterpret_cast<const uint8_t *>(sym), nl, nt, nc, s0, s1, s2, max_bins, nt,
+    return launch_cdf(reinterpret_cast<const uint8_t *>(sym), nullptr, 0, nl, nt, nc, s0, s1, s2, max_bins, nt,
                       reinterpret_cast<uint16_t *>(cdf), static_cast<hipStream_t>(stream));
 }
 
@@ -999,7 +1334,8 @@ int cg_encode_fast_new(const int16_t *cdf, int lp, const int8_t *sym, int64_t nl
     if (cap <= 0 || cap > INT_MAX) return fail(CG_ERR_ARG, "encode: bad output buffer length");
     const int block = pick_block(nc, lp);
     EncodeArgs a;
-    a.cdf = reinterpret_cast<const uint16_t *>(cdf);
+    memset(&a, 0, sizeof(a));
+    a.cdf = reinterpret_cast<uint16_t *>(const_cast<int16_t *>(cdf));      // only read here
     a.lp = lp;
     a.sym = reinterpret_cast<const uint8_t *>(sym);
     a.s0 = s0;
@@ -1013,14 +1349,15 @@ int cg_encode_fast_new(const int16_t *cdf, int lp, const int8_t *sym, int64_t nl
     a.lengths = lengths;
     a.status = nullptr;
     int64_t nblocks;
-    // nt == 0 still writes the two tail bits of every stream
+    // nt == 0 still writes the two closing bits of every stream
     if (int rc = make_grid(nl, nc, nt ? nt : 1, nt ? nt : 1, 1, block, a.sg, nblocks)) return rc;
     if (nt == 0) a.sg.g.T = 0;
     const size_t shmem = (size_t)lp * block * sizeof(uint32_t);
     const bool aligned = aligned_to(out, 4) && o0 % 4 == 0 && o1 % 4 == 0;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (aligned) encode_streams_kernel<true><<<dim3((unsigned)nblocks), dim3(block), shmem, st>>>(a);
-    else encode_streams_kernel<false><<<dim3((unsigned)nblocks), dim3(block), shmem, st>>>(a);
+    const dim3 grid((unsigned)nblocks), blk(block);
+    if (aligned) CG_DISPATCH_BS(block, (encode_streams_kernel<BS, true, false, false><<<grid, blk, shmem, st>>>(a)));
+    else CG_DISPATCH_BS(block, (encode_streams_kernel<BS, false, false, false><<<grid, blk, shmem, st>>>(a)));
     return check_launch("encode");
 }
 
@@ -1049,8 +1386,7 @@ int cg_decode_fast_new(const int16_t *cdf, int lp, const uint8_t *padded, int64_
     a.o2 = o2;
     int64_t nblocks;
     if (int rc = make_grid(nl, nc, nt, nt, 1, block, a.sg, nblocks)) return rc;
-    const size_t shmem = (size_t)lp * block * sizeof(uint32_t) + (lp + kSub) * sizeof(float);
-    return launch_decode_dt<SRC_PADDED, OUT_SYMBOLS>(a, nblocks, block, shmem, static_cast<hipStream_t>(stream));
+    return launch_decode_symbols<SRC_PADDED>(a, nblocks, block, static_cast<hipStream_t>(stream));
 }
 
 int cg_decode_fast_prefsum(const int16_t *cdf, int lp, const uint8_t *bytes, int64_t nbytes,
@@ -1067,6 +1403,7 @@ int cg_decode_fast_prefsum(const int16_t *cdf, int lp, const uint8_t *bytes, int
     a.cdf = reinterpret_cast<const uint16_t *>(cdf);
     a.lp = lp;
     a.bytes = bytes;
+    a.nbytes = nbytes;
     a.offsets = prefix;
     a.out_sym = out;
     a.o0 = o0;
@@ -1074,8 +1411,7 @@ int cg_decode_fast_prefsum(const int16_t *cdf, int lp, const uint8_t *bytes, int
     a.o2 = o2;
     int64_t nblocks;
     if (int rc = make_grid(nl, nc, nt, nt, 1, block, a.sg, nblocks)) return rc;
-    const size_t shmem = (size_t)lp * block * sizeof(uint32_t) + (lp + kSub) * sizeof(float);
-    return launch_decode_dt<SRC_PREFIX, OUT_SYMBOLS>(a, nblocks, block, shmem, static_cast<hipStream_t>(stream));
+    return launch_decode_symbols<SRC_PREFIX>(a, nblocks, block, static_cast<hipStream_t>(stream));
 }
 
 int cg_quantize_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D, int64_t sl,
@@ -1104,7 +1440,7 @@ size_t cg_encode_kv_workspace(int64_t L, int64_t T, int64_t C, int64_t chunk_tok
 {
     const int64_t nsub = cg_num_subchunks(T, chunk_tokens);
     const int64_t nstreams = nsub * 2 * L * C;
-    size_t total = align_up((size_t)(2 * L * T * C), 256);        // symbols
+    size_t total = align_up((size_t)nstreams * kSub, 256);        // symbols: a 256-token slot per stream
     total += align_up((size_t)nstreams * kStreamCap, 256);        // padded streams
     total += cg_scan_workspace(nstreams);
     return total;
@@ -1129,26 +1465,24 @@ int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int
     if (workspace_bytes < cg_encode_kv_workspace(L, T, C, chunk_tokens)) return fail(CG_ERR_WORKSPACE, "encode_kv: workspace too small");
     if (!aligned_to(workspace, 256)) return fail(CG_ERR_ARG, "encode_kv: workspace must be 256-byte aligned");
     hipStream_t s = static_cast<hipStream_t>(stream);
+    const int lp = max_bins + 1;
 
     uint8_t *ws = static_cast<uint8_t *>(workspace);
-    uint8_t *sym = ws;
-    ws += align_up((size_t)(rows * T * C), 256);
+    uint8_t *symbols = ws;
+    ws += align_up((size_t)nstreams * kSub, 256);
     uint8_t *padded = ws;
     ws += align_up((size_t)nstreams * kStreamCap, 256);
     void *scan_scratch = ws;
+    uint16_t *tables = reinterpret_cast<uint16_t *>(cdf);
 
     clear_status_kernel<<<1, 1, 0, s>>>(status);
-    if (int rc = launch_quantize(kv, kv_dt, L, T, H, D, sl, skv, st, sh, key_bins, value_bins, sym, maxima, s)) return rc;
-    if (int rc = launch_cdf(sym, rows, T, C, T * C, C, 1, max_bins, chunk_tokens, reinterpret_cast<uint16_t *>(cdf), s)) return rc;
 
-    const int block = pick_block(C, max_bins + 1);
+    const int block = pick_block(C, lp);
     EncodeArgs a;
-    a.cdf = reinterpret_cast<const uint16_t *>(cdf);
-    a.lp = max_bins + 1;
-    a.sym = sym;
-    a.s0 = T * C;
-    a.s1 = C;
-    a.s2 = 1;
+    memset(&a, 0, sizeof(a));
+    a.cdf = tables;
+    a.lp = lp;
+    a.nsub = nsub;
     a.out = padded;
     a.osub = rows * C * kStreamCap;
     a.o0 = C * kStreamCap;
@@ -1158,8 +1492,33 @@ int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int
     a.status = status;
     int64_t nblocks;
     if (int rc = make_grid(rows, C, T, chunk_tokens, nsub, block, a.sg, nblocks)) return rc;
-    const size_t shmem = (size_t)a.lp * block * sizeof(uint32_t);
-    encode_streams_kernel<true><<<dim3((unsigned)nblocks), dim3(block), shmem, s>>>(a);
+    const size_t shmem = (size_t)lp * block * sizeof(uint32_t);
+    const dim3 grid((unsigned)nblocks), blk(block);
+
+    const bool packed = kv_vectorizable(kv, D, C, sl, skv, st, sh) && C % 8 == 0;
+    if (packed) {
+        // four tokens per word, read by one lane per channel
+        uint32_t *sym4 = reinterpret_cast<uint32_t *>(symbols);
+        if (int rc = launch_quantize_pack(kv, kv_dt, L, T, H, D, sl, skv, st, sh, key_bins, value_bins, sym4,
+                                          maxima, nsub, chunk_tokens, s)) return rc;
+        a.sym4 = sym4;
+        if (chunk_tokens <= kSub) {
+            // one sub-chunk per chunk: the encoder builds the tables itself
+            CG_DISPATCH_BS(block, (encode_streams_kernel<BS, true, true, true><<<grid, blk, shmem, s>>>(a)));
+        } else {
+            if (int rc = launch_cdf(nullptr, sym4, nsub, rows, T, C, 0, 0, 0, max_bins, chunk_tokens, tables, s)) return rc;
+            CG_DISPATCH_BS(block, (encode_streams_kernel<BS, true, true, false><<<grid, blk, shmem, s>>>(a)));
+        }
+    } else {
+        // any shape or alignment: byte symbols [2L, T, C]
+        if (int rc = launch_quantize(kv, kv_dt, L, T, H, D, sl, skv, st, sh, key_bins, value_bins, symbols, maxima, s)) return rc;
+        if (int rc = launch_cdf(symbols, nullptr, 0, rows, T, C, T * C, C, 1, max_bins, chunk_tokens, tables, s)) return rc;
+        a.sym = symbols;
+        a.s0 = T * C;
+        a.s1 = C;
+        a.s2 = 1;
+        CG_DISPATCH_BS(block, (encode_streams_kernel<BS, true, false, false><<<grid, blk, shmem, s>>>(a)));
+    }
     if (int rc = check_launch("encode_kv")) return rc;
 
     if (int rc = launch_scan(lengths, nstreams, kStreamCap, offsets, scan_scratch, s)) return rc;
@@ -1191,6 +1550,7 @@ int cg_decode_kv(const int16_t *cdf, int max_bins, const void *maxima, int max_d
     a.cdf = reinterpret_cast<const uint16_t *>(cdf);
     a.lp = max_bins + 1;
     a.bytes = payload;
+    a.nbytes = payload_bytes;
     a.offsets = offsets;
     a.out_kv = static_cast<uint16_t *>(out);
     a.ol = ol;
@@ -1205,10 +1565,12 @@ int cg_decode_kv(const int16_t *cdf, int max_bins, const void *maxima, int max_d
     a.value_bins = value_bins;
     int64_t nblocks;
     if (int rc = make_grid(rows, C, T, chunk_tokens, nsub, block, a.sg, nblocks)) return rc;
-    const size_t shmem = (size_t)a.lp * block * sizeof(uint32_t) + (a.lp + kSub) * sizeof(float);
+    const size_t shmem = decode_shmem(a.lp, block);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (out_dt == CG_DT_BF16) return launch_decode_dt<SRC_OFFSETS, OUT_BF16>(a, nblocks, block, shmem, s);
-    return launch_decode_dt<SRC_OFFSETS, OUT_F16>(a, nblocks, block, shmem, s);
+    const dim3 grid((unsigned)nblocks);
+    if (out_dt == CG_DT_BF16) CG_DISPATCH_BS(block, (launch_decode_kv_log2<BS, OUT_BF16>(a, grid, shmem, s)));
+    else CG_DISPATCH_BS(block, (launch_decode_kv_log2<BS, OUT_F16>(a, grid, shmem, s)));
+    return check_launch("decode_kv");
 }
 
 }  // extern "C"

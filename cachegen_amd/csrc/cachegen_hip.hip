@@ -537,9 +537,10 @@ __device__ __forceinline__ StreamId locate(const StreamGrid &sg)
 
 // ---- encoder (enc_new.cu:21-97, 253-307) -------------------------------------------
 // Bits are collected MSB-first in a 32-bit accumulator and leave as big-endian words.
-// The E1/E2 run of a symbol is emitted at once: clz(low ^ high) leading bits agree, the
-// first of them is followed by the pending complements; the E3 run is the number of
-// positions below those where low has ones and high has zeros.  One combined shift by
+// The E1/E2 run of a symbol is emitted at once: the n1 = clz(low ^ high) leading bits
+// agree, and the pending complements go in after the first of them, which in arithmetic
+// is  bits + ((2^pend - 1) << (n1 - 1))  over n1 + pend bits.  The E3 run k is the number
+// of positions below those where low has ones and high has zeros.  One combined shift by
 // n = n1 + k renormalises low and high; n <= 18 for any table whose symbols all have
 // non-zero width, because the span stays above 2^30 between symbols.
 template <bool ALIGNED>
@@ -550,9 +551,16 @@ struct BitWriter {
     uint32_t acc;
     int nacc;
 
+    // the last words of a stream that does not fit its slot: keep what fits
+    __device__ __forceinline__ static void store_clipped(uint8_t *dst, int nbytes, int cap, uint32_t word)
+    {
+        for (int j = 0; j < 4; ++j)
+            if (nbytes + j < cap) dst[nbytes + j] = (uint8_t)(word >> (24 - 8 * j));
+    }
+
     __device__ __forceinline__ void store_word(uint32_t word)
     {
-        if (nbytes + 4 <= cap) {
+        if (__builtin_expect(nbytes + 4 <= cap, 1)) {
             if (ALIGNED) {
                 *reinterpret_cast<uint32_t *>(dst + nbytes) = __builtin_bswap32(word);
             } else {
@@ -562,34 +570,38 @@ struct BitWriter {
                 dst[nbytes + 3] = (uint8_t)word;
             }
         } else {
-            for (int j = 0; j < 4; ++j)
-                if (nbytes + j < cap) dst[nbytes + j] = (uint8_t)(word >> (24 - 8 * j));
+            store_clipped(dst, nbytes, cap, word);
         }
         nbytes += 4;
     }
 
-    // append the low m bits of v (v < 2^m), 1 <= m <= 32
+    // append the low m bits of v (v < 2^m), 0 <= m <= 32 (m = 0 needs v = 0)
     __device__ __forceinline__ void put(uint32_t v, int m)
     {
         const int tot = nacc + m;
-        if (tot < 32) {
-            acc = (acc << m) | v;
-            nacc = tot;
-        } else {
-            const uint32_t vl = v << (32 - m);
+        if (tot >= 32) {
+            const uint32_t vl = v << ((32 - m) & 31);
             store_word(__builtin_amdgcn_alignbit(acc, vl, (uint32_t)nacc));
             nacc = tot - 32;
             acc = v & ((1u << nacc) - 1u);
+        } else {
+            acc = (acc << m) | v;
+            nacc = tot;
         }
     }
 
-    __device__ __forceinline__ void run(uint32_t bit, uint32_t count)
+    // one bit, then `count` copies of its complement (any count): the general form of
+    // append_bit_and_pending (enc_new.cu:86-97); not on the common path
+    __device__ __forceinline__ void bit_and_run(uint32_t bit, uint32_t count)
     {
-        while (count > 0) {
-            const int take = count < 32u ? (int)count : 32;
-            const uint32_t ones = take == 32 ? 0xFFFFFFFFu : ((1u << take) - 1u);
-            put(bit ? ones : 0u, take);
-            count -= (uint32_t)take;
+        uint32_t pv = bit;
+        int pm = 1;
+        for (;;) {
+            put(pv, pm);
+            if (count == 0) break;
+            pm = count < 32u ? (int)count : 32;
+            pv = bit ? 0u : (pm == 32 ? 0xFFFFFFFFu : ((1u << pm) - 1u));
+            count -= (uint32_t)pm;
         }
     }
 
@@ -611,14 +623,14 @@ struct BitWriter {
 template <int BS, bool ALIGNED>
 struct RangeEncoder {
     const uint32_t *col;    // this lane's table column: entry e at col[e * BS]
-    uint32_t top;           // lp - 1: index of the table end (holds 2^16)
+    uint32_t smax;          // lp - 2: the largest symbol
     uint32_t low, high, pend;
     BitWriter<ALIGNED> w;
 
     __device__ __forceinline__ void init(const uint32_t *column, int lp, uint8_t *dst, int cap)
     {
         col = column;
-        top = (uint32_t)(lp - 1);
+        smax = (uint32_t)(lp - 2);
         low = 0;
         high = 0xFFFFFFFFu;
         pend = 0;
@@ -631,7 +643,7 @@ struct RangeEncoder {
 
     __device__ __forceinline__ void put_symbol(uint32_t s)
     {
-        s = s < top ? s : top - 1;                      // keep table reads inside the table
+        s = s < smax ? s : smax;                        // keep table reads inside the table
         const uint32_t r = high - low;
         const uint32_t rh = r >> 16, rl = r & 0xFFFFu;
         const uint32_t c_lo = col[s * BS];
@@ -644,19 +656,13 @@ struct RangeEncoder {
 
         const int n1 = __builtin_clz(low ^ high);       // low < high always
         if (n1 > 0) {
-            const uint32_t bits = low >> ((32 - n1) & 31);          // the n1 agreed bits
-            if (pend == 0) {
-                w.put(bits, n1);
-            } else if (pend + (uint32_t)n1 <= 32u) {
-                const uint32_t b = bits >> (n1 - 1);
-                const uint32_t head = ((1u << pend) - 1u) + b;       // b, then `pend` complements
-                const uint32_t rest = bits & ((1u << (n1 - 1)) - 1u);
-                w.put((head << (n1 - 1)) | rest, (int)pend + n1);
+            const uint32_t bits = low >> ((32 - n1) & 31);           // the n1 agreed bits
+            if (__builtin_expect(pend + (uint32_t)n1 > 32u, 0)) {
+                w.bit_and_run(bits >> (n1 - 1), pend);
+                w.put(bits & ((1u << (n1 - 1)) - 1u), n1 - 1);
             } else {
-                const uint32_t b = bits >> (n1 - 1);
-                w.put(b, 1);
-                w.run(1u - b, pend);
-                if (n1 > 1) w.put(bits & ((1u << (n1 - 1)) - 1u), n1 - 1);
+                const uint32_t fill = ((1u << (pend & 31)) - 1u) << (n1 - 1);
+                w.put(bits + fill, n1 + (int)pend);
             }
             pend = 0;
         }
@@ -670,9 +676,7 @@ struct RangeEncoder {
     __device__ __forceinline__ int finish()
     {
         pend += 1;
-        const uint32_t b = low < 0x40000000u ? 0u : 1u;
-        w.put(b, 1);
-        w.run(1u - b, pend);
+        w.bit_and_run(low < 0x40000000u ? 0u : 1u, pend);
         return w.finish();
     }
 };
@@ -777,47 +781,53 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
 // ---- decoder (dec_new.cu:35-71, 248-302) -------------------------------------------
 // The decoder tracks off = value - low, which every renormalisation step maps to
 // 2*off + next bit (E1/E2 and E3 alike), and finds the symbol as the largest m with
-// floor(span*cdf[m] / 2^16) <= off; that is the same m as the reference's search of
-// count = ((value-low+1)*2^16 - 1) / span in a strictly increasing table, without the
-// 64-bit divide.  The stream is read through aligned big-endian words with one raw word
-// in flight.  Bits past the end of a stream are whatever follows it in memory instead of
-// the reference's zeros (dec_new.cu:223-233): the coder's two closing bits place the
-// code value inside the final interval for every continuation, so the n symbols that
-// were encoded decode identically.  Loads never pass the end of the byte buffer.
+// T(m) = floor(span*cdf[m] / 2^16) <= off; that is the same m as the reference's search
+// of count = ((value-low+1)*2^16 - 1) / span in a strictly increasing table, without the
+// 64-bit divide.  For tables of 2^k symbols the search probes with the lower bound
+// (span >> 16) * cdf[m] <= T(m) (one multiply), which can only overshoot, and the result
+// is then walked back while the exact T(m) exceeds off (almost never).
+// The stream is read through aligned big-endian words with one raw word in flight.  Bits
+// past the end of a stream are whatever follows it in memory instead of the reference's
+// zeros (dec_new.cu:223-233): the coder's two closing bits place the code value inside
+// the final interval for every continuation, so the n symbols that were encoded decode
+// identically.  Word loads are clamped to the last word of the byte buffer.
 struct BitReader {
-    const uint32_t *words;   // aligned word holding the stream's first byte
-    uint32_t nwords_ok;      // words from `words` that lie inside the byte buffer
+    const uint8_t *base;     // 4-byte aligned, uniform over the block
+    uint32_t last;           // byte offset of the last word that may be read
+    uint32_t pos;            // byte offset of the next word to fetch
     uint32_t w0, w1, raw2;
     int c;                   // unread low bits of w0
-    uint32_t next;           // index of the next word to fetch
 
-    __device__ __forceinline__ uint32_t raw(uint32_t j) const { return j < nwords_ok ? words[j] : 0u; }
-
-    // position on the stream that begins at `begin`; `buf_end` is one past the last byte
-    // that may be read (rounded up to a word here); returns the stream's first 32 bits
-    __device__ __forceinline__ uint32_t start(const uint8_t *begin, const uint8_t *buf_end)
+    __device__ __forceinline__ uint32_t raw()
     {
-        const uint32_t skip = (uint32_t)(reinterpret_cast<uintptr_t>(begin) & 3u);
-        const uint8_t *aligned = begin - skip;
-        words = reinterpret_cast<const uint32_t *>(aligned);
-        const int64_t span_bytes = buf_end - aligned;
-        nwords_ok = span_bytes > 0 ? (uint32_t)((span_bytes + 3) >> 2) : 0u;
-        const uint32_t b0 = __builtin_bswap32(raw(0)), b1 = __builtin_bswap32(raw(1));
+        const uint32_t at = pos < last ? pos : last;
+        pos += 4;
+        return *reinterpret_cast<const uint32_t *>(base + at);
+    }
+
+    // position on the stream that begins `begin` bytes after `base`; returns its first 32 bits
+    __device__ __forceinline__ uint32_t start(const uint8_t *aligned_base, uint32_t last_word, uint32_t begin)
+    {
+        base = aligned_base;
+        last = last_word;
+        const uint32_t skip = begin & 3u;
+        pos = begin - skip;
+        const uint32_t b0 = __builtin_bswap32(raw()), b1 = __builtin_bswap32(raw());
+        const uint32_t r2 = raw(), r3 = raw();
         uint32_t first;
         if (skip == 0) {
             first = b0;
             w0 = b0;
             c = 0;
             w1 = b1;
-            raw2 = raw(2);
-            next = 3;
+            raw2 = r2;
+            pos -= 4;
         } else {
             c = 32 - (int)(skip * 8u);
             first = __builtin_amdgcn_alignbit(b0, b1, (uint32_t)c);
             w0 = b1;
-            w1 = __builtin_bswap32(raw(2));
-            raw2 = raw(3);
-            next = 4;
+            w1 = __builtin_bswap32(r2);
+            raw2 = r3;
         }
         return first;
     }
@@ -832,8 +842,7 @@ struct BitReader {
             w0 = w1;
             w1 = __builtin_bswap32(raw2);
             c += 32;
-            raw2 = raw(next);
-            next++;
+            raw2 = raw();
         }
         return off;
     }
@@ -845,12 +854,11 @@ enum { OUT_SYMBOLS = 0, OUT_F16 = 1, OUT_BF16 = 2 };
 struct DecodeArgs {
     const uint16_t *cdf;
     int32_t lp;
-    const uint8_t *bytes;       // payload, or padded buffer
-    int64_t nbytes;             // readable bytes from `bytes`
+    const uint8_t *bytes;       // payload or padded buffer, rounded down to a 4-byte boundary
+    uint32_t bytes_skew;        // bytes dropped by that rounding (0..3)
+    uint32_t last_word;         // byte offset from `bytes` of the last readable word
     const int64_t *offsets;     // SRC_OFFSETS: exclusive sums [nstreams+1]; SRC_PREFIX: inclusive sums
-    const int32_t *lengths;     // SRC_PADDED
     int64_t p0, p1;             // SRC_PADDED strides
-    int32_t cap;
     // OUT_SYMBOLS: out[row*o0 + token*o1 + channel*o2] uint8
     uint8_t *out_sym;
     int64_t o0, o1, o2;
@@ -894,23 +902,18 @@ __global__ __launch_bounds__(BS) void decode_streams_kernel(DecodeArgs a)
     }
     __syncthreads();
     if (!id.active) return;
+    uint32_t *col = tab + tid;
+    // the upper bound of the last symbol is 2^16, not the stored value (dec_new.cu:278)
+    col[(lp - 1) * BS] = 0x10000u;
 
     const int64_t stream = (id.sub * a.sg.rows + id.row) * a.sg.nc + id.ch;
-    const uint8_t *begin;
-    const uint8_t *buf_end;
-    if (SRC == SRC_OFFSETS) {
-        begin = a.bytes + a.offsets[stream];
-        buf_end = a.bytes + a.nbytes;
-    } else if (SRC == SRC_PREFIX) {
-        begin = a.bytes + (stream ? a.offsets[stream - 1] : 0);
-        buf_end = a.bytes + a.nbytes;
-    } else {
-        begin = a.bytes + id.row * a.p0 + id.ch * a.p1;
-        buf_end = begin + a.cap;
-    }
+    uint32_t begin;
+    if (SRC == SRC_OFFSETS) begin = (uint32_t)a.offsets[stream];
+    else if (SRC == SRC_PREFIX) begin = stream ? (uint32_t)a.offsets[stream - 1] : 0u;
+    else begin = (uint32_t)(id.row * a.p0 + id.ch * a.p1);
 
     BitReader rd;
-    uint32_t off = rd.start(begin, buf_end);
+    uint32_t off = rd.start(a.bytes, a.last_word, begin + a.bytes_skew);
     uint32_t low = 0, high = 0xFFFFFFFFu;
 
     uint8_t *osym = nullptr;
@@ -922,61 +925,78 @@ __global__ __launch_bounds__(BS) void decode_streams_kernel(DecodeArgs a)
         okv = a.out_kv + l * a.ol + kvi * a.okv + id.t0 * a.ot + h * a.oh + (id.ch - h * a.D);
     }
 
-    const uint32_t *col = tab + tid;
     int nsteps = 0;
     if (LOG2 < 0)
         while ((1 << nsteps) < lp - 1) ++nsteps;
 
-    for (int i = 0; i < id.n; ++i) {
-        const uint32_t r = high - low;
-        const uint32_t rh = r >> 16, rl = r & 0xFFFFu;
-        uint32_t sidx;                     // decoded symbol
-        uint32_t c_lo, c_hi;
-        if (LOG2 >= 0) {
-            uint32_t pos = 0;                  // element offset of the current entry in the column
-#pragma unroll
-            for (int step = (1 << LOG2) >> 1; step >= 1; step >>= 1) {
-                const uint32_t t = scale16(rh, rl, col[pos + step * BS]);
-                pos = (t <= off) ? pos + step * BS : pos;
-            }
-            sidx = pos / BS;
-            c_lo = col[pos];
-            c_hi = col[pos + BS];
-        } else {
-            int lo_i = 0, hi_i = lp - 1;
-            for (int step = 0; step < nsteps; ++step) {
-                const int mid = (lo_i + hi_i) >> 1;
-                const uint32_t t = scale16(rh, rl, col[mid * BS]);
-                const bool le = mid > 0 && t <= off;
-                lo_i = le ? mid : lo_i;
-                hi_i = le ? hi_i : mid;
-            }
-            sidx = (uint32_t)lo_i;
-            c_lo = col[lo_i * BS];
-            c_hi = col[lo_i * BS + BS];
-        }
-        if (OUT == OUT_SYMBOLS) {
-            osym[(int64_t)i * a.o1] = (uint8_t)sidx;
-        } else {
-            const float v = __fmul_rn(lut[sidx], rowmax[i]);
-            *okv = (uint16_t)(OUT == OUT_BF16 ? store16f<CG_DT_BF16>(v) : store16f<CG_DT_F16>(v));
-            okv += a.ot;
-        }
-        if (i == id.n - 1) break;                       // no update after the last symbol
-        const uint32_t t_lo = scale16(rh, rl, c_lo);
-        // the last symbol's upper bound is 2^16 (dec_new.cu:278): span * 2^16 >> 16 = span
-        const uint32_t t_hi_table = scale16(rh, rl, c_hi);
-        const uint32_t t_hi = sidx == (uint32_t)(lp - 2) ? r + 1u : t_hi_table;
-        high = low + t_hi - 1u;
-        low = low + t_lo;
-        off -= t_lo;
+    // LDS-typed views (32-bit addresses) of this lane's column, the quotient table and
+    // the row maxima
+    typedef __attribute__((address_space(3))) const uint32_t lds_u32;
+    typedef __attribute__((address_space(3))) const float lds_f32;
+    typedef __attribute__((address_space(3))) const char lds_char;
+    lds_u32 *const colp = (lds_u32 *)col;
+    lds_f32 *const lutp = (lds_f32 *)lut;
+    lds_f32 *rmp = (lds_f32 *)rowmax;
 
-        const int n1 = __builtin_clz(low ^ high);
-        const int k = __builtin_clz(~((low & ~high) << ((n1 + 1) & 31)));
-        const int n = (n1 + k) & 31;
-        low = (low << n) & 0x7FFFFFFFu;
-        high = (high << n) | 0x80000000u | ~(0xFFFFFFFFu << n);
-        off = rd.shift_in(off, n);
+    for (int i0 = 0; i0 < id.n; i0 += 4, rmp += 4) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int i = i0 + j;
+            if (i >= id.n) break;
+            const uint32_t r = high - low;
+            const uint32_t rh = r >> 16, rl = r & 0xFFFFu;
+            lds_u32 *p = colp;             // entry of the decoded symbol
+            uint32_t c_lo, t_lo;
+            if (LOG2 >= 0) {
+#pragma unroll
+                for (int step = (1 << LOG2) >> 1; step >= 1; step >>= 1) {
+                    const uint32_t t = __umul24(rh, p[step * BS]);
+                    p = (t <= off) ? p + step * BS : p;
+                }
+                for (;;) {
+                    c_lo = *p;
+                    t_lo = scale16(rh, rl, c_lo);
+                    if (__builtin_expect(t_lo <= off || p == colp, 1)) break;
+                    p -= BS;
+                }
+            } else {
+                int lo_i = 0, hi_i = lp - 1;
+                for (int step = 0; step < nsteps; ++step) {
+                    const int mid = (lo_i + hi_i) >> 1;
+                    const uint32_t t = scale16(rh, rl, colp[mid * BS]);
+                    const bool le = mid > 0 && t <= off;
+                    lo_i = le ? mid : lo_i;
+                    hi_i = le ? hi_i : mid;
+                }
+                p = colp + lo_i * BS;
+                c_lo = *p;
+                t_lo = scale16(rh, rl, c_lo);
+            }
+            // byte distance from the column start = symbol * BS * 4
+            const uint32_t sym4 = (uint32_t)((lds_char *)p - (lds_char *)colp) / BS;   // symbol * 4
+            if (OUT == OUT_SYMBOLS) {
+                osym[(int64_t)i * a.o1] = (uint8_t)(sym4 >> 2);
+            } else {
+                const float q = *(lds_f32 *)((lds_char *)lutp + sym4);
+                const float v = __fmul_rn(q, rmp[j]);
+                *okv = (uint16_t)(OUT == OUT_BF16 ? store16f<CG_DT_BF16>(v) : store16f<CG_DT_F16>(v));
+                okv += a.ot;
+            }
+            if (i == id.n - 1) break;                   // no update after the last symbol
+            const uint32_t c_hi = p[BS];
+            const uint32_t t_hi_table = scale16(rh, rl, c_hi);
+            const uint32_t t_hi = c_hi == 0x10000u ? r + 1u : t_hi_table;   // span * 2^16 >> 16 = span
+            high = low + t_hi - 1u;
+            low = low + t_lo;
+            off -= t_lo;
+
+            const int n1 = __builtin_clz(low ^ high);
+            const int k = __builtin_clz(~((low & ~high) << ((n1 + 1) & 31)));
+            const int n = (n1 + k) & 31;
+            low = (low << n) & 0x7FFFFFFFu;
+            high = (high << n) | 0x80000000u | ~(0xFFFFFFFFu << n);
+            off = rd.shift_in(off, n);
+        }
     }
 }
 
@@ -1265,6 +1285,19 @@ int launch_quantize_pack(const void *kv, int kv_dt, int64_t L, int64_t T, int64_
     return check_launch("quantize_pack");
 }
 
+// Describe the readable byte window [bytes, bytes + nbytes) to the bit reader, which
+// loads aligned words at 32-bit offsets from the window's 4-byte-aligned base.
+int set_byte_window(DecodeArgs &a, const uint8_t *bytes, int64_t nbytes, const char *what)
+{
+    if (nbytes <= 0) return fail(CG_ERR_ARG, "%s: empty byte buffer", what);
+    const uint32_t skew = (uint32_t)(reinterpret_cast<uintptr_t>(bytes) & 3u);
+    if (nbytes + skew > 0xFFFFFFF0ll) return fail(CG_ERR_ARG, "%s: byte buffers of 4 GiB or more must be decoded in pieces", what);
+    a.bytes = bytes - skew;
+    a.bytes_skew = skew;
+    a.last_word = (uint32_t)((skew + nbytes - 1) & ~3ll);
+    return CG_OK;
+}
+
 size_t decode_shmem(int lp, int block) { return (size_t)lp * block * sizeof(uint32_t) + (size_t)(lp + kSub) * sizeof(float); }
 
 template <int SRC>
@@ -1375,11 +1408,9 @@ int cg_decode_fast_new(const int16_t *cdf, int lp, const uint8_t *padded, int64_
     memset(&a, 0, sizeof(a));
     a.cdf = reinterpret_cast<const uint16_t *>(cdf);
     a.lp = lp;
-    a.bytes = padded;
-    a.lengths = lengths;
+    if (int rc = set_byte_window(a, padded, (nl - 1) * p0 + (nc - 1) * p1 + cap, "decode")) return rc;
     a.p0 = p0;
     a.p1 = p1;
-    a.cap = (int32_t)cap;
     a.out_sym = out;
     a.o0 = o0;
     a.o1 = o1;
@@ -1393,7 +1424,7 @@ int cg_decode_fast_prefsum(const int16_t *cdf, int lp, const uint8_t *bytes, int
                            const int64_t *prefix, int64_t nl, int64_t nt, int64_t nc, uint8_t *out,
                            int64_t o0, int64_t o1, int64_t o2, void *stream)
 {
-    if (!cdf || !prefix || !out || (!bytes && nbytes > 0)) return fail(CG_ERR_ARG, "decode: null pointer");
+    if (!cdf || !prefix || !out || !bytes) return fail(CG_ERR_ARG, "decode: null pointer");
     if (int rc = check_lp(lp, "decode")) return rc;
     if (nl <= 0 || nc <= 0 || nt <= 0) return fail(CG_ERR_ARG, "decode: empty input");
     if (nt > kSub) return fail(CG_ERR_ARG, "Number of tokens should be less than or equal to %d", kSub);
@@ -1402,8 +1433,7 @@ int cg_decode_fast_prefsum(const int16_t *cdf, int lp, const uint8_t *bytes, int
     memset(&a, 0, sizeof(a));
     a.cdf = reinterpret_cast<const uint16_t *>(cdf);
     a.lp = lp;
-    a.bytes = bytes;
-    a.nbytes = nbytes;
+    if (int rc = set_byte_window(a, bytes, nbytes, "decode")) return rc;
     a.offsets = prefix;
     a.out_sym = out;
     a.o0 = o0;
@@ -1535,7 +1565,7 @@ int cg_decode_kv(const int16_t *cdf, int max_bins, const void *maxima, int max_d
                  int64_t chunk_tokens, void *out, int out_dt, int64_t ol, int64_t okv, int64_t ot,
                  int64_t oh, void *stream)
 {
-    if (!cdf || !maxima || !offsets || !key_bins || !value_bins || !out || (!payload && payload_bytes > 0))
+    if (!cdf || !maxima || !offsets || !key_bins || !value_bins || !out || !payload)
         return fail(CG_ERR_ARG, "decode_kv: null pointer");
     if (int rc = check_dt(max_dt, "decode_kv")) return rc;
     if (int rc = check_dt(out_dt, "decode_kv")) return rc;
@@ -1549,8 +1579,7 @@ int cg_decode_kv(const int16_t *cdf, int max_bins, const void *maxima, int max_d
     memset(&a, 0, sizeof(a));
     a.cdf = reinterpret_cast<const uint16_t *>(cdf);
     a.lp = max_bins + 1;
-    a.bytes = payload;
-    a.nbytes = payload_bytes;
+    if (int rc = set_byte_window(a, payload, payload_bytes, "decode_kv")) return rc;
     a.offsets = offsets;
     a.out_kv = static_cast<uint16_t *>(out);
     a.ol = ol;

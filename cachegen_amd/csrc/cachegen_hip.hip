@@ -545,33 +545,34 @@ __device__ __forceinline__ StreamId locate(const StreamGrid &sg)
 // non-zero width, because the span stays above 2^30 between symbols.
 template <bool ALIGNED>
 struct BitWriter {
-    uint8_t *dst;
+    uint8_t *wptr;          // where the next word goes
     int cap;
     int nbytes;
     uint32_t acc;
     int nacc;
 
     // the last words of a stream that does not fit its slot: keep what fits
-    __device__ __forceinline__ static void store_clipped(uint8_t *dst, int nbytes, int cap, uint32_t word)
+    __device__ __forceinline__ void store_clipped(uint32_t word)
     {
         for (int j = 0; j < 4; ++j)
-            if (nbytes + j < cap) dst[nbytes + j] = (uint8_t)(word >> (24 - 8 * j));
+            if (nbytes + j < cap) wptr[j] = (uint8_t)(word >> (24 - 8 * j));
     }
 
     __device__ __forceinline__ void store_word(uint32_t word)
     {
         if (__builtin_expect(nbytes + 4 <= cap, 1)) {
             if (ALIGNED) {
-                *reinterpret_cast<uint32_t *>(dst + nbytes) = __builtin_bswap32(word);
+                *reinterpret_cast<uint32_t *>(wptr) = __builtin_bswap32(word);
             } else {
-                dst[nbytes + 0] = (uint8_t)(word >> 24);
-                dst[nbytes + 1] = (uint8_t)(word >> 16);
-                dst[nbytes + 2] = (uint8_t)(word >> 8);
-                dst[nbytes + 3] = (uint8_t)word;
+                wptr[0] = (uint8_t)(word >> 24);
+                wptr[1] = (uint8_t)(word >> 16);
+                wptr[2] = (uint8_t)(word >> 8);
+                wptr[3] = (uint8_t)word;
             }
         } else {
-            store_clipped(dst, nbytes, cap, word);
+            store_clipped(word);
         }
+        wptr += 4;
         nbytes += 4;
     }
 
@@ -610,8 +611,8 @@ struct BitWriter {
     {
         if (nacc > 0) {
             uint32_t r = acc << (32 - nacc);
-            for (int left = nacc; left > 0; left -= 8) {
-                if (nbytes < cap) dst[nbytes] = (uint8_t)(r >> 24);
+            for (int left = nacc, j = 0; left > 0; left -= 8, ++j) {
+                if (nbytes < cap) wptr[j] = (uint8_t)(r >> 24);
                 nbytes++;
                 r <<= 8;
             }
@@ -634,7 +635,7 @@ struct RangeEncoder {
         low = 0;
         high = 0xFFFFFFFFu;
         pend = 0;
-        w.dst = dst;
+        w.wptr = dst;
         w.cap = cap;
         w.nbytes = 0;
         w.acc = 0;
@@ -688,8 +689,8 @@ struct EncodeArgs {
     int64_t s0, s1, s2;
     const uint32_t *sym4;   // or packed symbols
     int64_t nsub;
-    uint8_t *out;           // out[sub*osub + row*o0 + channel*o1 + byte]
-    int64_t osub, o0, o1;
+    uint8_t *out;           // out[row*o0 + channel*o1 + byte], or one `cap`-byte slot per
+    int64_t o0, o1;         // stream in stream order (SLOTS)
     int32_t cap;
     int32_t *lengths;       // [sub][row][channel]
     int32_t *status;        // may be null
@@ -698,7 +699,8 @@ struct EncodeArgs {
 
 // PACKED: symbols come from sym4.  FUSE_CDF (PACKED only, one sub-chunk per chunk): the
 // block first builds its own tables from the same words and writes them out.
-template <int BS, bool ALIGNED, bool PACKED, bool FUSE_CDF>
+// SLOTS: stream g of the launch is written to out[g * cap ...] (the fused path's scratch).
+template <int BS, bool ALIGNED, bool PACKED, bool FUSE_CDF, bool SLOTS>
 __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
 {
     extern __shared__ uint32_t tab[];
@@ -712,19 +714,31 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
     const int nwords = (id.n + 3) >> 2;
     if (PACKED) wp = a.sym4 + ((id.row * a.nsub + id.sub) * kWordsPerSub) * a.sg.nc + id.ch;
 
+    // PACKED: the lane's whole sub-chunk (64 words = 256 symbols) is loaded once into
+    // registers and indexed by the (uniform) loop counter, so the coding loop has no loads
+    // to wait for and its stores never hold it up.
+    typedef uint32_t words32 __attribute__((ext_vector_type(32)));
+    words32 words_a, words_b;          // words 0..31 and 32..63 of the sub-chunk
+    if (PACKED) {
+#pragma unroll
+        for (int w = 0; w < 32; ++w) {
+            words_a[w] = (id.active && w < nwords) ? wp[(int64_t)w * a.sg.nc] : 0u;
+            words_b[w] = (id.active && w + 32 < nwords) ? wp[(int64_t)(w + 32) * a.sg.nc] : 0u;
+        }
+    }
+
     if (FUSE_CDF) {
         for (int i = 0; i < lp; ++i) col[i * BS] = 0;
         if (id.active) {
             const uint32_t smax = (uint32_t)(lp - 2);
-            for (int w0 = 0; w0 < nwords; w0 += 4) {
-                uint32_t v[4];
+#pragma unroll 1
+            for (int w = 0; w < nwords; ++w) {
+                const uint32_t v = w < 32 ? words_a[w & 31] : words_b[w & 31];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) v[j] = (w0 + j < nwords) ? wp[(int64_t)(w0 + j) * a.sg.nc] : 0u;
-#pragma unroll
-                for (int j = 0; j < 16; ++j) {
-                    uint32_t s = (v[j >> 2] >> (8 * (j & 3))) & 0xFFu;
+                for (int j = 0; j < 4; ++j) {
+                    uint32_t s = (v >> (8 * j)) & 0xFFu;
                     s = s < smax ? s : smax;
-                    if (w0 * 4 + j < id.n) atomicAdd(&col[(s + 1) * BS], 1u);
+                    if (w * 4 + j < id.n) atomicAdd(&col[(s + 1) * BS], 1u);
                 }
             }
             normalize_column_total<BS>(col, lp, lp - 1, (uint32_t)id.n);
@@ -741,21 +755,16 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
     col[(lp - 1) * BS] = 0x10000u;
 
     RangeEncoder<BS, ALIGNED> enc;
-    enc.init(col, lp, a.out + id.sub * a.osub + id.row * a.o0 + id.ch * a.o1, a.cap);
+    const int64_t stream = (id.sub * a.sg.rows + id.row) * a.sg.nc + id.ch;
+    enc.init(col, lp, SLOTS ? a.out + stream * a.cap : a.out + id.row * a.o0 + id.ch * a.o1, a.cap);
 
     if (PACKED) {
-        uint32_t nxt[4];
+#pragma unroll 1
+        for (int w = 0; w < nwords; ++w) {
+            const uint32_t v = w < 32 ? words_a[w & 31] : words_b[w & 31];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) nxt[j] = (j < nwords) ? wp[(int64_t)j * a.sg.nc] : 0u;
-        for (int w0 = 0; w0 < nwords; w0 += 4) {
-            uint32_t cur[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) cur[j] = nxt[j];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) nxt[j] = (w0 + 4 + j < nwords) ? wp[(int64_t)(w0 + 4 + j) * a.sg.nc] : 0u;
-#pragma unroll
-            for (int j = 0; j < 16; ++j)
-                if (w0 * 4 + j < id.n) enc.put_symbol((cur[j >> 2] >> (8 * (j & 3))) & 0xFFu);
+            for (int j = 0; j < 4; ++j)
+                if (w * 4 + j < id.n) enc.put_symbol((v >> (8 * j)) & 0xFFu);
         }
     } else {
         const uint8_t *sp = a.sym + id.row * a.s0 + id.t0 * a.s1 + id.ch * a.s2;
@@ -774,7 +783,7 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
         }
     }
     const int len = enc.finish();
-    a.lengths[(id.sub * a.sg.rows + id.row) * a.sg.nc + id.ch] = len;
+    a.lengths[stream] = len;
     if (len > a.cap && a.status) atomicOr(a.status, 1);
 }
 
@@ -1081,37 +1090,66 @@ __global__ __launch_bounds__(kScanThreads) void scan_apply_kernel(
 }
 
 // ------------------------------------------------------------------------------------
-// collect_bytes (encoder.py:209-222): each wavefront moves 64 streams from their padded
-// slots to their final offsets, one stream at a time with all lanes copying.
+// collect_bytes (encoder.py:209-222), output-centric: a block owns 256 consecutive
+// streams, i.e. one contiguous range of the payload.  Every thread assembles aligned
+// 32-bit words of that range: it finds the stream of the word's first byte by binary
+// search over the block's offsets (in LDS); a word that lies inside one stream is two
+// aligned loads from that stream's slot and a funnel shift, a word that straddles streams
+// or the ends of the range is gathered and stored byte by byte, so neighbouring blocks
+// never write the same byte.  All positions are 32-bit offsets from the range's start.
 // ------------------------------------------------------------------------------------
+constexpr int kCompactStreams = 256;
+
 __global__ __launch_bounds__(256) void compact_streams_kernel(
-    const uint8_t *__restrict__ padded, int32_t cap, const int32_t *__restrict__ lengths,
-    const int64_t *__restrict__ offsets, int64_t nstreams, uint8_t *__restrict__ payload,
-    int64_t payload_cap, int32_t *status)
+    const uint8_t *__restrict__ slots, int32_t cap, const int64_t *__restrict__ offsets,
+    int64_t nstreams, uint8_t *__restrict__ payload, int64_t payload_cap, int32_t skew, int32_t *status)
 {
-    const int lane = threadIdx.x & 63;
-    const int64_t first = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * 64;
-    if (first >= nstreams) return;
-    const int64_t mine = first + lane;
-    int my_len = 0;
-    int64_t my_off = 0;
-    if (mine < nstreams) {
-        my_len = lengths[mine];
-        my_len = my_len < 0 ? 0 : (my_len > cap ? cap : my_len);
-        my_off = offsets[mine];
+    __shared__ int32_t rel[kCompactStreams + 1];       // stream offsets relative to the block's first byte
+    const int tid = threadIdx.x;
+    const int64_t sbase = (int64_t)blockIdx.x * kCompactStreams;
+    const int count = (nstreams - sbase < kCompactStreams) ? (int)(nstreams - sbase) : kCompactStreams;
+    const int64_t o0 = offsets[sbase];
+    for (int i = tid; i <= kCompactStreams; i += 256)
+        rel[i] = (int32_t)(offsets[sbase + (i < count ? i : count)] - o0);
+    __syncthreads();
+    const int total = rel[count];
+    if (o0 + total > payload_cap) {                    // never write past the caller's buffer
+        if (tid == 0 && status) atomicOr(status, 2);
+        return;
     }
-    const int count = (nstreams - first < 64) ? (int)(nstreams - first) : 64;
-    bool spilled = false;
-    for (int s = 0; s < count; ++s) {
-        const int len = __shfl(my_len, s, 64);
-        const int64_t off = __shfl(my_off, s, 64);
-        const uint8_t *src = padded + (first + s) * (int64_t)cap;
-        for (int j = lane; j < len; j += 64) {
-            if (off + j < payload_cap) payload[off + j] = src[j];
-            else spilled = true;
+    const uint8_t *src = slots + sbase * (int64_t)cap;
+    uint8_t *dst = payload + o0;
+    // words are aligned in memory: `lead` bytes of the first word lie before the range
+    const int lead = (int)((o0 + skew) & 3);
+    const int nwords = (lead + total + 3) >> 2;
+    int nsteps = 0;
+    while ((1 << nsteps) < count) ++nsteps;
+    for (int w = tid; w < nwords; w += 256) {
+        const int p0 = 4 * w - lead;                   // may be negative for w = 0
+        const int pfirst = p0 < 0 ? 0 : p0;
+        const int pend = p0 + 4 < total ? p0 + 4 : total;
+        int lo = 0, hi = count - 1;                    // largest s with rel[s] <= pfirst
+        for (int step = 0; step < nsteps; ++step) {
+            const int mid = (lo + hi + 1) >> 1;
+            const bool le = rel[mid] <= pfirst;
+            lo = le ? mid : lo;
+            hi = le ? hi : mid - 1;
+        }
+        int s = lo;
+        if (pend - pfirst == 4 && pfirst + 3 < rel[s + 1]) {
+            const int q = pfirst - rel[s];
+            const uint8_t *slot = src + s * cap;       // 32-bit offset: 256 streams * cap bytes
+            const int at = q & ~3, sh = (q & 3) * 8;
+            const uint32_t w_lo = *reinterpret_cast<const uint32_t *>(slot + at);
+            const uint32_t w_hi = (sh != 0) ? *reinterpret_cast<const uint32_t *>(slot + at + 4) : 0u;
+            *reinterpret_cast<uint32_t *>(dst + p0) = __builtin_amdgcn_alignbit(w_hi, w_lo, (uint32_t)sh);
+        } else {
+            for (int p = pfirst; p < pend; ++p) {
+                while (p >= rel[s + 1]) ++s;           // streams are at least one byte long
+                dst[p] = src[s * cap + (p - rel[s])];
+            }
         }
     }
-    if (spilled && status) atomicOr(status, 2);
 }
 
 __global__ void clear_status_kernel(int32_t *status) { *status = 0; }
@@ -1375,7 +1413,6 @@ int cg_encode_fast_new(const int16_t *cdf, int lp, const int8_t *sym, int64_t nl
     a.s1 = s1;
     a.s2 = s2;
     a.out = out;
-    a.osub = 0;
     a.o0 = o0;
     a.o1 = o1;
     a.cap = (int32_t)cap;
@@ -1389,8 +1426,8 @@ int cg_encode_fast_new(const int16_t *cdf, int lp, const int8_t *sym, int64_t nl
     const bool aligned = aligned_to(out, 4) && o0 % 4 == 0 && o1 % 4 == 0;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const dim3 grid((unsigned)nblocks), blk(block);
-    if (aligned) CG_DISPATCH_BS(block, (encode_streams_kernel<BS, true, false, false><<<grid, blk, shmem, st>>>(a)));
-    else CG_DISPATCH_BS(block, (encode_streams_kernel<BS, false, false, false><<<grid, blk, shmem, st>>>(a)));
+    if (aligned) CG_DISPATCH_BS(block, (encode_streams_kernel<BS, true, false, false, false><<<grid, blk, shmem, st>>>(a)));
+    else CG_DISPATCH_BS(block, (encode_streams_kernel<BS, false, false, false, false><<<grid, blk, shmem, st>>>(a)));
     return check_launch("encode");
 }
 
@@ -1471,7 +1508,7 @@ size_t cg_encode_kv_workspace(int64_t L, int64_t T, int64_t C, int64_t chunk_tok
     const int64_t nsub = cg_num_subchunks(T, chunk_tokens);
     const int64_t nstreams = nsub * 2 * L * C;
     size_t total = align_up((size_t)nstreams * kSub, 256);        // symbols: a 256-token slot per stream
-    total += align_up((size_t)nstreams * kStreamCap, 256);        // padded streams
+    total += align_up((size_t)nstreams * kStreamCap, 256);        // encoder scratch: a slot per stream
     total += cg_scan_workspace(nstreams);
     return total;
 }
@@ -1500,7 +1537,7 @@ int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int
     uint8_t *ws = static_cast<uint8_t *>(workspace);
     uint8_t *symbols = ws;
     ws += align_up((size_t)nstreams * kSub, 256);
-    uint8_t *padded = ws;
+    uint8_t *scratch = ws;     // one kStreamCap-byte slot per stream
     ws += align_up((size_t)nstreams * kStreamCap, 256);
     void *scan_scratch = ws;
     uint16_t *tables = reinterpret_cast<uint16_t *>(cdf);
@@ -1513,10 +1550,7 @@ int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int
     a.cdf = tables;
     a.lp = lp;
     a.nsub = nsub;
-    a.out = padded;
-    a.osub = rows * C * kStreamCap;
-    a.o0 = C * kStreamCap;
-    a.o1 = kStreamCap;
+    a.out = scratch;
     a.cap = kStreamCap;
     a.lengths = lengths;
     a.status = status;
@@ -1534,10 +1568,10 @@ int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int
         a.sym4 = sym4;
         if (chunk_tokens <= kSub) {
             // one sub-chunk per chunk: the encoder builds the tables itself
-            CG_DISPATCH_BS(block, (encode_streams_kernel<BS, true, true, true><<<grid, blk, shmem, s>>>(a)));
+            CG_DISPATCH_BS(block, (encode_streams_kernel<BS, true, true, true, true><<<grid, blk, shmem, s>>>(a)));
         } else {
             if (int rc = launch_cdf(nullptr, sym4, nsub, rows, T, C, 0, 0, 0, max_bins, chunk_tokens, tables, s)) return rc;
-            CG_DISPATCH_BS(block, (encode_streams_kernel<BS, true, true, false><<<grid, blk, shmem, s>>>(a)));
+            CG_DISPATCH_BS(block, (encode_streams_kernel<BS, true, true, false, true><<<grid, blk, shmem, s>>>(a)));
         }
     } else {
         // any shape or alignment: byte symbols [2L, T, C]
@@ -1547,15 +1581,16 @@ int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int
         a.s0 = T * C;
         a.s1 = C;
         a.s2 = 1;
-        CG_DISPATCH_BS(block, (encode_streams_kernel<BS, true, false, false><<<grid, blk, shmem, s>>>(a)));
+        CG_DISPATCH_BS(block, (encode_streams_kernel<BS, true, false, false, true><<<grid, blk, shmem, s>>>(a)));
     }
     if (int rc = check_launch("encode_kv")) return rc;
 
     if (int rc = launch_scan(lengths, nstreams, kStreamCap, offsets, scan_scratch, s)) return rc;
-    const int64_t cblocks = ceil_div(nstreams, 256);
+    const int64_t cblocks = ceil_div(nstreams, kCompactStreams);
     if (cblocks > INT_MAX) return fail(CG_ERR_ARG, "encode_kv: too many streams");
-    compact_streams_kernel<<<dim3((unsigned)cblocks), dim3(256), 0, s>>>(padded, kStreamCap, lengths, offsets,
-                                                                      nstreams, payload, payload_cap, status);
+    compact_streams_kernel<<<dim3((unsigned)cblocks), dim3(256), 0, s>>>(
+        scratch, kStreamCap, offsets, nstreams, payload, payload_cap,
+        (int32_t)(reinterpret_cast<uintptr_t>(payload) & 3u), status);
     return check_launch("compact");
 }
 

@@ -113,13 +113,25 @@ __device__ __forceinline__ uint32_t store16f(float f)
     return DT == CG_DT_BF16 ? float_to_bf16_bits(f) : float_to_f16_bits(f);
 }
 
+// 24-bit multiply, low 32 bits of the product, as an unsigned value (HIP's __umul24 returns
+// int, which would turn a following >> into an arithmetic shift).
+__device__ __forceinline__ uint32_t mul24(uint32_t a, uint32_t b) { return (uint32_t)__umul24(a, b); }
+
 // floor(span * c / 2^16) for span = r + 1 (rh = r >> 16, rl = r & 0xffff) and a table
 // value c <= 0xffff, on the full-rate 24-bit multiplier: span*c = rh*c*2^16 + (rl+1)*c.
 // This is `(span * c) >> precision` of enc_new.cu:272-273 / dec_new.cu:280-281.
 __device__ __forceinline__ uint32_t scale16(uint32_t rh, uint32_t rl, uint32_t c)
 {
-    const uint32_t lowpart = __umul24(rl, c) + c;
-    return __umul24(rh, c) + (lowpart >> 16);
+    const uint32_t lowpart = mul24(rl, c) + c;
+    return mul24(rh, c) + (lowpart >> 16);
+}
+
+// The same product from the span itself (sh = span >> 16, sl = span & 0xffff), valid for
+// every span below 2^32 and every c up to and including 2^16 (where it returns the span):
+// span*c = sh*c*2^16 + sl*c.
+__device__ __forceinline__ uint32_t scale_span(uint32_t sh, uint32_t sl, uint32_t c)
+{
+    return mul24(sh, c) + (mul24(sl, c) >> 16);
 }
 
 // ------------------------------------------------------------------------------------
@@ -621,11 +633,15 @@ struct BitWriter {
     }
 };
 
+// The coder state is (low, span) with span = high - low + 1 held modulo 2^32: 0 stands for
+// the full range 2^32 (the initial state, and any later interval that is exactly a binary
+// fraction), where floor(span * c / 2^16) is simply c << 16.  Renormalising by n bits maps
+// span to span << n for E1/E2 and E3 steps alike.
 template <int BS, bool ALIGNED>
 struct RangeEncoder {
     const uint32_t *col;    // this lane's table column: entry e at col[e * BS]
     uint32_t smax;          // lp - 2: the largest symbol
-    uint32_t low, high, pend;
+    uint32_t low, span, pend;
     BitWriter<ALIGNED> w;
 
     __device__ __forceinline__ void init(const uint32_t *column, int lp, uint8_t *dst, int cap)
@@ -633,7 +649,7 @@ struct RangeEncoder {
         col = column;
         smax = (uint32_t)(lp - 2);
         low = 0;
-        high = 0xFFFFFFFFu;
+        span = 0;
         pend = 0;
         w.wptr = dst;
         w.cap = cap;
@@ -645,15 +661,19 @@ struct RangeEncoder {
     __device__ __forceinline__ void put_symbol(uint32_t s)
     {
         s = s < smax ? s : smax;                        // keep table reads inside the table
-        const uint32_t r = high - low;
-        const uint32_t rh = r >> 16, rl = r & 0xFFFFu;
         const uint32_t c_lo = col[s * BS];
-        const uint32_t c_hi = col[s * BS + BS];
-        const uint32_t t_lo = scale16(rh, rl, c_lo);
-        const uint32_t t_hi_table = scale16(rh, rl, c_hi);
-        const uint32_t t_hi = c_hi == 0x10000u ? r + 1u : t_hi_table;
-        high = low + t_hi - 1u;
-        low = low + t_lo;
+        const uint32_t c_hi = col[s * BS + BS];         // 2^16 for the last symbol
+        uint32_t t_lo, width;
+        if (__builtin_expect(span == 0, 0)) {
+            t_lo = c_lo << 16;
+            width = (c_hi - c_lo) << 16;
+        } else {
+            const uint32_t sh = span >> 16, sl = span & 0xFFFFu;
+            t_lo = scale_span(sh, sl, c_lo);
+            width = scale_span(sh, sl, c_hi) - t_lo;
+        }
+        low += t_lo;
+        const uint32_t high = low + width - 1u;
 
         const int n1 = __builtin_clz(low ^ high);       // low < high always
         if (n1 > 0) {
@@ -671,7 +691,7 @@ struct RangeEncoder {
         const int n = (n1 + k) & 31;
         pend += (uint32_t)k;
         low = (low << n) & 0x7FFFFFFFu;
-        high = (high << n) | 0x80000000u | ~(0xFFFFFFFFu << n);
+        span = width << n;
     }
 
     __device__ __forceinline__ int finish()
@@ -923,7 +943,7 @@ __global__ __launch_bounds__(BS) void decode_streams_kernel(DecodeArgs a)
 
     BitReader rd;
     uint32_t off = rd.start(a.bytes, a.last_word, begin + a.bytes_skew);
-    uint32_t low = 0, high = 0xFFFFFFFFu;
+    uint32_t low = 0, span = 0;        // span modulo 2^32: 0 is the full range (see RangeEncoder)
 
     uint8_t *osym = nullptr;
     uint16_t *okv = nullptr;
@@ -952,34 +972,55 @@ __global__ __launch_bounds__(BS) void decode_streams_kernel(DecodeArgs a)
         for (int j = 0; j < 4; ++j) {
             const int i = i0 + j;
             if (i >= id.n) break;
-            const uint32_t r = high - low;
-            const uint32_t rh = r >> 16, rl = r & 0xFFFFu;
             lds_u32 *p = colp;             // entry of the decoded symbol
-            uint32_t c_lo, t_lo;
-            if (LOG2 >= 0) {
+            uint32_t t_lo, width;
+            if (__builtin_expect(span == 0, 0)) {
+                // full range: T(m) = cdf[m] << 16, so compare table values with off >> 16
+                const uint32_t key = off >> 16;
+                if (LOG2 >= 0) {
 #pragma unroll
-                for (int step = (1 << LOG2) >> 1; step >= 1; step >>= 1) {
-                    const uint32_t t = __umul24(rh, p[step * BS]);
-                    p = (t <= off) ? p + step * BS : p;
+                    for (int step = (1 << LOG2) >> 1; step >= 1; step >>= 1)
+                        p = (p[step * BS] <= key) ? p + step * BS : p;
+                } else {
+                    int lo_i = 0, hi_i = lp - 1;
+                    for (int step = 0; step < nsteps; ++step) {
+                        const int mid = (lo_i + hi_i) >> 1;
+                        const bool le = mid > 0 && colp[mid * BS] <= key;
+                        lo_i = le ? mid : lo_i;
+                        hi_i = le ? hi_i : mid;
+                    }
+                    p = colp + lo_i * BS;
                 }
-                for (;;) {
-                    c_lo = *p;
-                    t_lo = scale16(rh, rl, c_lo);
-                    if (__builtin_expect(t_lo <= off || p == colp, 1)) break;
-                    p -= BS;
-                }
+                const uint32_t c_lo = *p;
+                t_lo = c_lo << 16;
+                width = (p[BS] - c_lo) << 16;
             } else {
-                int lo_i = 0, hi_i = lp - 1;
-                for (int step = 0; step < nsteps; ++step) {
-                    const int mid = (lo_i + hi_i) >> 1;
-                    const uint32_t t = scale16(rh, rl, colp[mid * BS]);
-                    const bool le = mid > 0 && t <= off;
-                    lo_i = le ? mid : lo_i;
-                    hi_i = le ? hi_i : mid;
+                const uint32_t sh = span >> 16, sl = span & 0xFFFFu;
+                if (LOG2 >= 0) {
+                    // probe with the lower bound sh * c <= T(c); it can only overshoot
+#pragma unroll
+                    for (int step = (1 << LOG2) >> 1; step >= 1; step >>= 1) {
+                        const uint32_t t = mul24(sh, p[step * BS]);
+                        p = (t <= off) ? p + step * BS : p;
+                    }
+                    t_lo = scale_span(sh, sl, *p);
+                    while (__builtin_expect(t_lo > off && p != colp, 0)) {
+                        p -= BS;
+                        t_lo = scale_span(sh, sl, *p);
+                    }
+                } else {
+                    int lo_i = 0, hi_i = lp - 1;
+                    for (int step = 0; step < nsteps; ++step) {
+                        const int mid = (lo_i + hi_i) >> 1;
+                        const uint32_t t = scale_span(sh, sl, colp[mid * BS]);
+                        const bool le = mid > 0 && t <= off;
+                        lo_i = le ? mid : lo_i;
+                        hi_i = le ? hi_i : mid;
+                    }
+                    p = colp + lo_i * BS;
+                    t_lo = scale_span(sh, sl, *p);
                 }
-                p = colp + lo_i * BS;
-                c_lo = *p;
-                t_lo = scale16(rh, rl, c_lo);
+                width = scale_span(sh, sl, p[BS]) - t_lo;
             }
             // byte distance from the column start = symbol * BS * 4
             const uint32_t sym4 = (uint32_t)((lds_char *)p - (lds_char *)colp) / BS;   // symbol * 4
@@ -992,18 +1033,14 @@ __global__ __launch_bounds__(BS) void decode_streams_kernel(DecodeArgs a)
                 okv += a.ot;
             }
             if (i == id.n - 1) break;                   // no update after the last symbol
-            const uint32_t c_hi = p[BS];
-            const uint32_t t_hi_table = scale16(rh, rl, c_hi);
-            const uint32_t t_hi = c_hi == 0x10000u ? r + 1u : t_hi_table;   // span * 2^16 >> 16 = span
-            high = low + t_hi - 1u;
-            low = low + t_lo;
+            low += t_lo;
             off -= t_lo;
-
+            const uint32_t high = low + width - 1u;
             const int n1 = __builtin_clz(low ^ high);
             const int k = __builtin_clz(~((low & ~high) << ((n1 + 1) & 31)));
             const int n = (n1 + k) & 31;
             low = (low << n) & 0x7FFFFFFFu;
-            high = (high << n) | 0x80000000u | ~(0xFFFFFFFFu << n);
+            span = width << n;
             off = rd.shift_in(off, n);
         }
     }

@@ -391,33 +391,6 @@ __device__ __forceinline__ void normalize_column(uint32_t *col, int lp, int max_
     }
 }
 
-// The same when every one of `total` tokens was counted (1 <= total <= 65535, uniform
-// over the block): the divide becomes a shift or a float estimate corrected exactly.
-template <int BS>
-__device__ __forceinline__ void normalize_column_total(uint32_t *col, int lp, int max_bins, uint32_t total)
-{
-    uint32_t running = 0;
-    for (int i = 1; i < lp; ++i) {
-        running += col[i * BS];
-        col[i * BS] = running;
-    }
-    const uint32_t scale = 0xFFFFu - (uint32_t)max_bins;
-    if ((total & (total - 1)) == 0) {
-        const int sh = 31 - __builtin_clz(total);
-        for (int i = 0; i < lp; ++i) col[i * BS] = ((scale * col[i * BS]) >> sh) + (uint32_t)i;
-    } else {
-        const float inv = __fdiv_rn(1.0f, (float)total);
-        for (int i = 0; i < lp; ++i) {
-            const uint32_t x = scale * col[i * BS];              // < 2^32, quotient < 2^16
-            uint32_t q = (uint32_t)((float)x * inv);
-            int32_t rem = (int32_t)(x - q * total);
-            if (rem < 0) { q--; rem += (int32_t)total; }
-            if (rem >= (int32_t)total) q++;
-            col[i * BS] = q + (uint32_t)i;
-        }
-    }
-}
-
 // Write the block's tables tab[entry * BS + lane] to cdf[lane][entry], coalesced.
 template <int BS>
 __device__ __forceinline__ void write_tables(const uint32_t *tab, uint16_t *cdf, int lp, int64_t ch0, int64_t nc)
@@ -439,6 +412,59 @@ __device__ __forceinline__ void stage_tables(uint32_t *tab, const uint16_t *cdf,
     for (int i = threadIdx.x; i < total; i += BS) {
         const int c = i / lp, e = i - c * lp;
         tab[e * BS + c] = cdf[i];
+    }
+}
+
+// The stream kernels keep their tables in LDS as 16-bit entries tab[entry * BS + lane]
+// (half the footprint, twice the resident waves).  The end of a table, 2^16, does not fit
+// and is substituted where the last symbol's upper bound is read.
+template <int BS>
+__device__ __forceinline__ void stage_tables16(uint16_t *tab, const uint16_t *cdf, int lp, int64_t ch0, int64_t nc)
+{
+    const int64_t nvalid = (nc - ch0 < BS) ? (nc - ch0) : BS;
+    const int total = (int)nvalid * lp;
+    for (int i = threadIdx.x; i < total; i += BS) {
+        const int c = i / lp, e = i - c * lp;
+        tab[e * BS + c] = cdf[i];
+    }
+}
+
+template <int BS>
+__device__ __forceinline__ void write_tables16(const uint16_t *tab, uint16_t *cdf, int lp, int64_t ch0, int64_t nc)
+{
+    const int64_t nvalid = (nc - ch0 < BS) ? (nc - ch0) : BS;
+    const int total = (int)nvalid * lp;
+    for (int i = threadIdx.x; i < total; i += BS) {
+        const int c = i / lp, e = i - c * lp;
+        cdf[i] = tab[e * BS + c];
+    }
+}
+
+// Running sum and normalisation of one lane's 16-bit column of counts when every one of
+// `total` tokens was counted (1 <= total <= 65535, uniform over the block): the divide of
+// cal_cdf.cu:11-14 becomes a shift or a float estimate corrected exactly.
+template <int BS>
+__device__ __forceinline__ void normalize_column16(uint16_t *col, int lp, int max_bins, uint32_t total)
+{
+    const uint32_t scale = 0xFFFFu - (uint32_t)max_bins;
+    uint32_t running = 0;
+    if ((total & (total - 1)) == 0) {
+        const int sh = 31 - __builtin_clz(total);
+        for (int i = 0; i < lp; ++i) {
+            running += col[i * BS];
+            col[i * BS] = (uint16_t)(((scale * running) >> sh) + (uint32_t)i);
+        }
+    } else {
+        const float inv = __fdiv_rn(1.0f, (float)total);
+        for (int i = 0; i < lp; ++i) {
+            running += col[i * BS];
+            const uint32_t x = scale * running;                  // < 2^32, quotient < 2^16
+            uint32_t q = (uint32_t)((float)x * inv);
+            int32_t rem = (int32_t)(x - q * total);
+            if (rem < 0) { q--; rem += (int32_t)total; }
+            if (rem >= (int32_t)total) q++;
+            col[i * BS] = (uint16_t)(q + (uint32_t)i);
+        }
     }
 }
 
@@ -639,12 +665,12 @@ struct BitWriter {
 // span to span << n for E1/E2 and E3 steps alike.
 template <int BS, bool ALIGNED>
 struct RangeEncoder {
-    const uint32_t *col;    // this lane's table column: entry e at col[e * BS]
+    const uint16_t *col;    // this lane's table column: entry e at col[e * BS]
     uint32_t smax;          // lp - 2: the largest symbol
     uint32_t low, span, pend;
     BitWriter<ALIGNED> w;
 
-    __device__ __forceinline__ void init(const uint32_t *column, int lp, uint8_t *dst, int cap)
+    __device__ __forceinline__ void init(const uint16_t *column, int lp, uint8_t *dst, int cap)
     {
         col = column;
         smax = (uint32_t)(lp - 2);
@@ -662,7 +688,8 @@ struct RangeEncoder {
     {
         s = s < smax ? s : smax;                        // keep table reads inside the table
         const uint32_t c_lo = col[s * BS];
-        const uint32_t c_hi = col[s * BS + BS];         // 2^16 for the last symbol
+        const uint32_t c_next = col[s * BS + BS];
+        const uint32_t c_hi = s == smax ? 0x10000u : c_next;    // the table ends at 2^16 (enc_new.cu:270)
         uint32_t t_lo, width;
         if (__builtin_expect(span == 0, 0)) {
             t_lo = c_lo << 16;
@@ -723,12 +750,12 @@ struct EncodeArgs {
 template <int BS, bool ALIGNED, bool PACKED, bool FUSE_CDF, bool SLOTS>
 __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
 {
-    extern __shared__ uint32_t tab[];
+    extern __shared__ uint16_t tab[];
     const int tid = threadIdx.x;
     const StreamId id = locate<BS>(a.sg);
     const int lp = a.lp;
     const int64_t ch0 = id.ch - tid;
-    uint32_t *col = tab + tid;
+    uint16_t *col = tab + tid;
     uint16_t *cdf_block = a.cdf + ((id.chunk * a.sg.rows + id.row) * a.sg.nc + ch0) * lp;
     const uint32_t *wp = nullptr;
     const int nwords = (id.n + 3) >> 2;
@@ -758,21 +785,18 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
                 for (int j = 0; j < 4; ++j) {
                     uint32_t s = (v >> (8 * j)) & 0xFFu;
                     s = s < smax ? s : smax;
-                    if (w * 4 + j < id.n) atomicAdd(&col[(s + 1) * BS], 1u);
+                    if (w * 4 + j < id.n) col[(s + 1) * BS]++;      // the column is this lane's own
                 }
             }
-            normalize_column_total<BS>(col, lp, lp - 1, (uint32_t)id.n);
+            normalize_column16<BS>(col, lp, lp - 1, (uint32_t)id.n);
         }
         __syncthreads();
-        write_tables<BS>(tab, cdf_block, lp, ch0, a.sg.nc);
-        __syncthreads();
+        write_tables16<BS>(tab, cdf_block, lp, ch0, a.sg.nc);
     } else {
-        stage_tables<BS>(tab, cdf_block, lp, ch0, a.sg.nc);
+        stage_tables16<BS>(tab, cdf_block, lp, ch0, a.sg.nc);
         __syncthreads();
     }
     if (!id.active) return;
-    // the upper bound of the last symbol is 2^16, not the stored value (enc_new.cu:270)
-    col[(lp - 1) * BS] = 0x10000u;
 
     RangeEncoder<BS, ALIGNED> enc;
     const int64_t stream = (id.sub * a.sg.rows + id.row) * a.sg.nc + id.ch;
@@ -911,11 +935,11 @@ __global__ __launch_bounds__(BS) void decode_streams_kernel(DecodeArgs a)
     const int tid = threadIdx.x;
     const StreamId id = locate<BS>(a.sg);
     const int lp = LOG2 >= 0 ? (1 << LOG2) + 1 : a.lp;
-    uint32_t *tab = smem;
-    float *lut = reinterpret_cast<float *>(smem + lp * BS);   // (s - C) / C per symbol
+    uint16_t *tab = reinterpret_cast<uint16_t *>(smem);
+    float *lut = reinterpret_cast<float *>(smem + (lp * BS + 1) / 2);   // (s - C) / C per symbol
     float *rowmax = lut + lp;                                 // one per token of the sub-chunk
     const int64_t ch0 = id.ch - tid;
-    stage_tables<BS>(tab, a.cdf + ((id.chunk * a.sg.rows + id.row) * a.sg.nc + ch0) * lp, lp, ch0, a.sg.nc);
+    stage_tables16<BS>(tab, a.cdf + ((id.chunk * a.sg.rows + id.row) * a.sg.nc + ch0) * lp, lp, ch0, a.sg.nc);
     int64_t kvi = 0, l = 0;
     if (OUT != OUT_SYMBOLS) {
         kvi = id.row / a.L;
@@ -931,9 +955,7 @@ __global__ __launch_bounds__(BS) void decode_streams_kernel(DecodeArgs a)
     }
     __syncthreads();
     if (!id.active) return;
-    uint32_t *col = tab + tid;
-    // the upper bound of the last symbol is 2^16, not the stored value (dec_new.cu:278)
-    col[(lp - 1) * BS] = 0x10000u;
+    uint16_t *col = tab + tid;
 
     const int64_t stream = (id.sub * a.sg.rows + id.row) * a.sg.nc + id.ch;
     uint32_t begin;
@@ -960,10 +982,11 @@ __global__ __launch_bounds__(BS) void decode_streams_kernel(DecodeArgs a)
 
     // LDS-typed views (32-bit addresses) of this lane's column, the quotient table and
     // the row maxima
-    typedef __attribute__((address_space(3))) const uint32_t lds_u32;
+    typedef __attribute__((address_space(3))) const uint16_t lds_u16;
     typedef __attribute__((address_space(3))) const float lds_f32;
     typedef __attribute__((address_space(3))) const char lds_char;
-    lds_u32 *const colp = (lds_u32 *)col;
+    lds_u16 *const colp = (lds_u16 *)col;
+    lds_u16 *const plast = colp + (lp - 2) * BS;      // entry of the last symbol
     lds_f32 *const lutp = (lds_f32 *)lut;
     lds_f32 *rmp = (lds_f32 *)rowmax;
 
@@ -972,7 +995,7 @@ __global__ __launch_bounds__(BS) void decode_streams_kernel(DecodeArgs a)
         for (int j = 0; j < 4; ++j) {
             const int i = i0 + j;
             if (i >= id.n) break;
-            lds_u32 *p = colp;             // entry of the decoded symbol
+            lds_u16 *p = colp;             // entry of the decoded symbol
             uint32_t t_lo, width;
             if (__builtin_expect(span == 0, 0)) {
                 // full range: T(m) = cdf[m] << 16, so compare table values with off >> 16
@@ -992,8 +1015,9 @@ __global__ __launch_bounds__(BS) void decode_streams_kernel(DecodeArgs a)
                     p = colp + lo_i * BS;
                 }
                 const uint32_t c_lo = *p;
+                const uint32_t c_hi = p == plast ? 0x10000u : (uint32_t)p[BS];   // dec_new.cu:278
                 t_lo = c_lo << 16;
-                width = (p[BS] - c_lo) << 16;
+                width = (c_hi - c_lo) << 16;
             } else {
                 const uint32_t sh = span >> 16, sl = span & 0xFFFFu;
                 if (LOG2 >= 0) {
@@ -1020,10 +1044,11 @@ __global__ __launch_bounds__(BS) void decode_streams_kernel(DecodeArgs a)
                     p = colp + lo_i * BS;
                     t_lo = scale_span(sh, sl, *p);
                 }
-                width = scale_span(sh, sl, p[BS]) - t_lo;
+                const uint32_t c_hi = p == plast ? 0x10000u : (uint32_t)p[BS];   // dec_new.cu:278
+                width = scale_span(sh, sl, c_hi) - t_lo;
             }
-            // byte distance from the column start = symbol * BS * 4
-            const uint32_t sym4 = (uint32_t)((lds_char *)p - (lds_char *)colp) / BS;   // symbol * 4
+            // byte distance from the column start = symbol * BS * 2
+            const uint32_t sym4 = (uint32_t)((lds_char *)p - (lds_char *)colp) / (BS / 2);   // symbol * 4
             if (OUT == OUT_SYMBOLS) {
                 osym[(int64_t)i * a.o1] = (uint8_t)(sym4 >> 2);
             } else {
@@ -1199,8 +1224,7 @@ __global__ void clear_status_kernel(int32_t *status) { *status = 0; }
 int pick_block(int64_t nc, int lp)
 {
     int block = 256;
-    if (lp > 40) block = 128;
-    if (lp > 80) block = 64;
+    if (lp > 80) block = 128;
     while (block > 64 && nc <= block / 2) block /= 2;
     return block;
 }
@@ -1373,7 +1397,7 @@ int set_byte_window(DecodeArgs &a, const uint8_t *bytes, int64_t nbytes, const c
     return CG_OK;
 }
 
-size_t decode_shmem(int lp, int block) { return (size_t)lp * block * sizeof(uint32_t) + (size_t)(lp + kSub) * sizeof(float); }
+size_t decode_shmem(int lp, int block) { return align_up((size_t)lp * block * sizeof(uint16_t), 4) + (size_t)(lp + kSub) * sizeof(float); }
 
 template <int SRC>
 int launch_decode_symbols(const DecodeArgs &a, int64_t nblocks, int block, hipStream_t stream)
@@ -1459,7 +1483,7 @@ int cg_encode_fast_new(const int16_t *cdf, int lp, const int8_t *sym, int64_t nl
     // nt == 0 still writes the two closing bits of every stream
     if (int rc = make_grid(nl, nc, nt ? nt : 1, nt ? nt : 1, 1, block, a.sg, nblocks)) return rc;
     if (nt == 0) a.sg.g.T = 0;
-    const size_t shmem = (size_t)lp * block * sizeof(uint32_t);
+    const size_t shmem = (size_t)lp * block * sizeof(uint16_t);
     const bool aligned = aligned_to(out, 4) && o0 % 4 == 0 && o1 % 4 == 0;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const dim3 grid((unsigned)nblocks), blk(block);
@@ -1593,7 +1617,7 @@ int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int
     a.status = status;
     int64_t nblocks;
     if (int rc = make_grid(rows, C, T, chunk_tokens, nsub, block, a.sg, nblocks)) return rc;
-    const size_t shmem = (size_t)lp * block * sizeof(uint32_t);
+    const size_t shmem = (size_t)lp * block * sizeof(uint16_t);
     const dim3 grid((unsigned)nblocks), blk(block);
 
     const bool packed = kv_vectorizable(kv, D, C, sl, skv, st, sh) && C % 8 == 0;

@@ -761,31 +761,33 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
     const int nwords = (id.n + 3) >> 2;
     if (PACKED) wp = a.sym4 + ((id.row * a.nsub + id.sub) * kWordsPerSub) * a.sg.nc + id.ch;
 
-    // PACKED: the lane's whole sub-chunk (64 words = 256 symbols) is loaded once into
-    // registers and indexed by the (uniform) loop counter, so the coding loop has no loads
-    // to wait for and its stores never hold it up.
+    // PACKED: half a sub-chunk (32 words = 128 symbols) at a time is loaded into registers
+    // and indexed by the (uniform) loop counter, so the coding loop has no loads to wait
+    // for and its stores never hold it up.
     typedef uint32_t words32 __attribute__((ext_vector_type(32)));
-    words32 words_a, words_b;          // words 0..31 and 32..63 of the sub-chunk
-    if (PACKED) {
+    words32 words;
+    auto load_half = [&](int h) {
 #pragma unroll
-        for (int w = 0; w < 32; ++w) {
-            words_a[w] = (id.active && w < nwords) ? wp[(int64_t)w * a.sg.nc] : 0u;
-            words_b[w] = (id.active && w + 32 < nwords) ? wp[(int64_t)(w + 32) * a.sg.nc] : 0u;
-        }
-    }
+        for (int w = 0; w < 32; ++w)
+            words[w] = (id.active && h * 32 + w < nwords) ? wp[(int64_t)(h * 32 + w) * a.sg.nc] : 0u;
+    };
 
     if (FUSE_CDF) {
         for (int i = 0; i < lp; ++i) col[i * BS] = 0;
         if (id.active) {
             const uint32_t smax = (uint32_t)(lp - 2);
+            for (int h = 0; h * 32 < nwords; ++h) {
+                load_half(h);
+                const int wn = nwords - h * 32 < 32 ? nwords - h * 32 : 32;
 #pragma unroll 1
-            for (int w = 0; w < nwords; ++w) {
-                const uint32_t v = w < 32 ? words_a[w & 31] : words_b[w & 31];
+                for (int w = 0; w < wn; ++w) {
+                    const uint32_t v = words[w];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    uint32_t s = (v >> (8 * j)) & 0xFFu;
-                    s = s < smax ? s : smax;
-                    if (w * 4 + j < id.n) col[(s + 1) * BS]++;      // the column is this lane's own
+                    for (int j = 0; j < 4; ++j) {
+                        uint32_t s = (v >> (8 * j)) & 0xFFu;
+                        s = s < smax ? s : smax;
+                        if ((h * 32 + w) * 4 + j < id.n) col[(s + 1) * BS]++;   // the column is this lane's own
+                    }
                 }
             }
             normalize_column16<BS>(col, lp, lp - 1, (uint32_t)id.n);
@@ -803,12 +805,16 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
     enc.init(col, lp, SLOTS ? a.out + stream * a.cap : a.out + id.row * a.o0 + id.ch * a.o1, a.cap);
 
     if (PACKED) {
+        for (int h = 0; h * 32 < nwords; ++h) {
+            load_half(h);
+            const int wn = nwords - h * 32 < 32 ? nwords - h * 32 : 32;
 #pragma unroll 1
-        for (int w = 0; w < nwords; ++w) {
-            const uint32_t v = w < 32 ? words_a[w & 31] : words_b[w & 31];
+            for (int w = 0; w < wn; ++w) {
+                const uint32_t v = words[w];
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                if (w * 4 + j < id.n) enc.put_symbol((v >> (8 * j)) & 0xFFu);
+                for (int j = 0; j < 4; ++j)
+                    if ((h * 32 + w) * 4 + j < id.n) enc.put_symbol((v >> (8 * j)) & 0xFFu);
+            }
         }
     } else {
         const uint8_t *sp = a.sym + id.row * a.s0 + id.t0 * a.s1 + id.ch * a.s2;

@@ -1465,7 +1465,7 @@ int cg_encode_fast_new(const int16_t *cdf, int lp, const int8_t *sym, int64_t nl
                        int64_t s0, int64_t s1, int64_t s2, uint8_t *out, int64_t cap, int64_t o0,
                        int64_t o1, int32_t *lengths, void *stream)
 {
-    if (!cdf || !sym || !out || !lengths) return fail(CG_ERR_ARG, "encode: null pointer");
+    if (!cdf || (!sym && nt > 0) || !out || !lengths) return fail(CG_ERR_ARG, "encode: null pointer");
     if (int rc = check_lp(lp, "encode")) return rc;
     if (nl <= 0 || nc <= 0 || nt < 0) return fail(CG_ERR_ARG, "encode: empty input");
     if (nt > kSub) return fail(CG_ERR_ARG, "Number of tokens should be less than or equal to %d", kSub);

@@ -1,0 +1,125 @@
+"""Benchmark-size runs on the GPU, checked through size-independent properties (the oracle
+is too slow at these sizes): reconstruction within half a quantization step, idempotence of
+re-encoding the decoded cache, independence of chunks (a chunk encoded alone equals its slice
+of the batched result), agreement of the fused decoder with the four-entry-point path, and
+table invariants."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _bins(model, monkeypatch=None):
+    from cachegen_amd.serde import cachegen_basics as B
+    cfg = B.CacheGenConfig.from_model_name(model)
+    return B.make_key_bins(cfg).to(DEV), B.make_value_bins(cfg).to(DEV)
+
+
+@pytest.fixture(scope="module")
+def mistral_8k():
+    """Benchmark config 2: 32 layers x {K,V} x 8192 tokens x 8 heads x 128, table per 256 tokens."""
+    from cachegen_amd import codec
+    from cachegen_amd.kvgen import make_kv
+    kv = make_kv(32, 8192, 8, 128, seed=1236, device=DEV)
+    kb, vb = _bins("lmsys/longchat-7b-16k")
+    enc = codec.encode_kv(kv, kb, vb, chunk_tokens=256)
+    enc.check()
+    out = codec.decode_encoded(enc, kb, vb, fmt="vllm", out_dtype=torch.float16)
+    torch.cuda.synchronize()
+    return kv, kb, vb, enc, out
+
+
+def test_full_size_round_trip_within_half_step(mistral_8k):
+    kv, kb, vb, enc, out = mistral_8k
+    L, _, T, H, D = kv.shape
+    maxq = torch.stack([kb, vb], dim=1).div(2, rounding_mode="floor").sub(1)[:, :, None, None]
+    for l0 in range(0, L, 8):                       # in slices to bound memory
+        x = kv[l0:l0 + 8].reshape(8, 2, T, H * D).float()
+        y = out[l0:l0 + 8].reshape(8, 2, T, H * D).float()
+        step = x.abs().amax(dim=-1, keepdim=True) / maxq[l0:l0 + 8]
+        assert bool(((x - y).abs() <= 0.52 * step).all())
+    # row maxima are exact copies of the input's
+    assert torch.equal(enc.maxima, kv.reshape(L, 2, T, H * D).abs().amax(dim=-1).permute(1, 0, 2))
+
+
+def test_full_size_tables_and_lengths_are_well_formed(mistral_8k):
+    kv, kb, vb, enc, out = mistral_8k
+    cdf = enc.cdf.view(torch.uint16).to(torch.int32)
+    assert int(cdf[..., 0].max()) == 0 and int(cdf[..., -1].min()) == 65535
+    assert bool((cdf[..., 1:] > cdf[..., :-1]).all())
+    assert int(enc.lengths.min()) >= 1 and int(enc.lengths.max()) <= 256
+    off = enc.offsets
+    assert int(off[0]) == 0 and bool((off[1:] - off[:-1] == enc.lengths.flatten()).all())
+    assert enc.total_bytes() == int(enc.lengths.sum())
+
+
+def test_full_size_reencoding_is_idempotent(mistral_8k):
+    from cachegen_amd import codec
+    kv, kb, vb, enc, out = mistral_8k
+    again = codec.encode_kv(out, kb, vb, chunk_tokens=256)
+    again.check()
+    n = enc.total_bytes()
+    assert again.total_bytes() == n
+    assert torch.equal(again.lengths, enc.lengths)
+    assert torch.equal(again.cdf, enc.cdf)
+    assert torch.equal(again.payload[:n], enc.payload[:n])
+
+
+def test_full_size_chunks_are_independent(mistral_8k):
+    """Chunk k encoded on its own (one `to_bytes` call of the reference) is byte-identical to
+    its slice of the batched encode."""
+    from cachegen_amd import codec
+    kv, kb, vb, enc, out = mistral_8k
+    bounds = enc.sub_boundaries()
+    for k in (0, 13, 31):
+        one = codec.encode_kv(kv[:, :, k * 256:(k + 1) * 256], kb, vb, chunk_tokens=256)
+        one.check()
+        cdf, mk, mv, subs = enc.chunk(k, bounds)
+        assert torch.equal(one.cdf[0], cdf)
+        assert torch.equal(one.lengths[0], subs[0][1])
+        assert torch.equal(one.payload[:one.total_bytes()], subs[0][0])
+        assert torch.equal(one.maxima[0, :, :, None], mk)
+
+
+def test_full_size_fused_decode_agrees_with_entry_points(mistral_8k):
+    """Symbols from decode_fast_prefsum on a chunk's slice, dequantized with plain tensor ops,
+    equal the fused decoder's output (float32 ops rounded one by one in both)."""
+    from cachegen_amd import codec, torchac_hip as tac
+    from cachegen_amd.serde.cachegen_decoder import do_dequantize
+    kv, kb, vb, enc, out = mistral_8k
+    bounds = enc.sub_boundaries()
+    k = 7
+    cdf, mk, mv, subs = enc.chunk(k, bounds)
+    data, lengths, n = subs[0]
+    prefix = codec.scan_lengths(lengths)[1:].view(lengths.shape)
+    sym = torch.zeros((64, n, 1024), dtype=torch.uint8, device=DEV)
+    tac.decode_fast_prefsum(cdf, data, prefix, sym)
+    key = do_dequantize(sym[:32].float(), kb, mk).to(torch.float16)
+    val = do_dequantize(sym[32:].float(), vb, mv).to(torch.float16)
+    got = out[:, :, k * 256:(k + 1) * 256].reshape(32, 2, n, 1024)
+    assert torch.equal(got[:, 0], key) and torch.equal(got[:, 1], val)
+    # and the quantizer's symbols for that chunk are what was coded
+    qsym, _ = codec.quantize_kv(kv[:, :, k * 256:(k + 1) * 256], kb, vb)
+    assert torch.equal(qsym, sym)
+
+
+def test_llama70b_table_long_chunks_round_trip():
+    """Benchmark config 4's geometry at reduced length: 80 layers, 1500-token chunks cut into
+    5 x 256 + 220 token streams, 70B bins table."""
+    from cachegen_amd import codec
+    from cachegen_amd.kvgen import make_kv
+    L, T = 80, 3200
+    kv = make_kv(L, T, 8, 128, seed=1238, device=DEV)
+    kb, vb = _bins("Yukang/LongAlpaca-70B-16k")
+    enc = codec.encode_kv(kv, kb, vb, chunk_tokens=1500)
+    enc.check()
+    assert enc.lengths.shape[0] == 6 + 6 + 1 and enc.cdf.shape[0] == 3
+    out = codec.decode_encoded(enc, kb, vb, fmt="vllm", out_dtype=torch.float16)
+    again = codec.encode_kv(out, kb, vb, chunk_tokens=1500)
+    n = enc.total_bytes()
+    assert again.total_bytes() == n and torch.equal(again.payload[:n], enc.payload[:n])
+    x, y = kv.reshape(L, 2, T, 1024).float(), out.reshape(L, 2, T, 1024).float()
+    maxq = torch.stack([kb, vb], dim=1).div(2, rounding_mode="floor").sub(1)[:, :, None, None]
+    assert bool(((x - y).abs() <= 0.52 * x.abs().amax(dim=-1, keepdim=True) / maxq).all())

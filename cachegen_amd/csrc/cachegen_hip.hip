@@ -851,9 +851,9 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
 // the final interval for every continuation, so the n symbols that were encoded decode
 // identically.  Word loads are clamped to the last word of the byte buffer.
 struct BitReader {
-    const uint8_t *base;     // 4-byte aligned, uniform over the block
-    uint32_t last;           // byte offset of the last word that may be read
-    uint32_t pos;            // byte offset of the next word to fetch
+    const uint8_t *base;     // the aligned word holding the stream's first byte
+    uint32_t last;           // byte offset from `base` of the last word that may be read
+    uint32_t pos;            // byte offset from `base` of the next word to fetch
     uint32_t w0, w1, raw2;
     int c;                   // unread low bits of w0
 
@@ -864,13 +864,16 @@ struct BitReader {
         return *reinterpret_cast<const uint32_t *>(base + at);
     }
 
-    // position on the stream that begins `begin` bytes after `base`; returns its first 32 bits
-    __device__ __forceinline__ uint32_t start(const uint8_t *aligned_base, uint32_t last_word, uint32_t begin)
+    // position on the stream that begins `begin` bytes after the 4-byte aligned `window`,
+    // whose last readable word is at byte offset `last_word`; returns the first 32 bits
+    __device__ __forceinline__ uint32_t start(const uint8_t *window, int64_t last_word, int64_t begin)
     {
-        base = aligned_base;
-        last = last_word;
-        const uint32_t skip = begin & 3u;
-        pos = begin - skip;
+        const uint32_t skip = (uint32_t)begin & 3u;
+        const int64_t first_word = begin - skip;
+        base = window + first_word;
+        const int64_t room = last_word - first_word;
+        last = room < 0 ? 0u : (room > 0xFFFFFFF0ll ? 0xFFFFFFF0u : (uint32_t)room);
+        pos = 0;
         const uint32_t b0 = __builtin_bswap32(raw()), b1 = __builtin_bswap32(raw());
         const uint32_t r2 = raw(), r3 = raw();
         uint32_t first;
@@ -915,7 +918,7 @@ struct DecodeArgs {
     int32_t lp;
     const uint8_t *bytes;       // payload or padded buffer, rounded down to a 4-byte boundary
     uint32_t bytes_skew;        // bytes dropped by that rounding (0..3)
-    uint32_t last_word;         // byte offset from `bytes` of the last readable word
+    int64_t last_word;          // byte offset from `bytes` of the last readable word
     const int64_t *offsets;     // SRC_OFFSETS: exclusive sums [nstreams+1]; SRC_PREFIX: inclusive sums
     int64_t p0, p1;             // SRC_PADDED strides
     // OUT_SYMBOLS: out[row*o0 + token*o1 + channel*o2] uint8
@@ -964,10 +967,10 @@ __global__ __launch_bounds__(BS) void decode_streams_kernel(DecodeArgs a)
     uint16_t *col = tab + tid;
 
     const int64_t stream = (id.sub * a.sg.rows + id.row) * a.sg.nc + id.ch;
-    uint32_t begin;
-    if (SRC == SRC_OFFSETS) begin = (uint32_t)a.offsets[stream];
-    else if (SRC == SRC_PREFIX) begin = stream ? (uint32_t)a.offsets[stream - 1] : 0u;
-    else begin = (uint32_t)(id.row * a.p0 + id.ch * a.p1);
+    int64_t begin;
+    if (SRC == SRC_OFFSETS) begin = a.offsets[stream];
+    else if (SRC == SRC_PREFIX) begin = stream ? a.offsets[stream - 1] : 0;
+    else begin = id.row * a.p0 + id.ch * a.p1;
 
     BitReader rd;
     uint32_t off = rd.start(a.bytes, a.last_word, begin + a.bytes_skew);
@@ -1402,10 +1405,9 @@ int set_byte_window(DecodeArgs &a, const uint8_t *bytes, int64_t nbytes, const c
 {
     if (nbytes <= 0) return fail(CG_ERR_ARG, "%s: empty byte buffer", what);
     const uint32_t skew = (uint32_t)(reinterpret_cast<uintptr_t>(bytes) & 3u);
-    if (nbytes + skew > 0xFFFFFFF0ll) return fail(CG_ERR_ARG, "%s: byte buffers of 4 GiB or more must be decoded in pieces", what);
     a.bytes = bytes - skew;
     a.bytes_skew = skew;
-    a.last_word = (uint32_t)((skew + nbytes - 1) & ~3ll);
+    a.last_word = (skew + nbytes - 1) & ~3ll;
     return CG_OK;
 }
 

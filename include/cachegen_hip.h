@@ -79,7 +79,7 @@ int cg_decode_fast_new(const int16_t *cdf, int lp, const uint8_t *padded, int64_
 
 /* torchac_cuda.decode_fast_prefsum (dec_new.cu:403-479): streams concatenated in
  * (layer, channel) order.
- * bytes    device uint8 [nbytes], nbytes < 4 GiB; the decoder loads whole aligned 32-bit
+ * bytes    device uint8 [nbytes]; the decoder loads whole aligned 32-bit
  *          words, so up to 3 bytes on either side of the buffer (inside the same aligned
  *          words) are read but never used
  * prefix   device int64 [nl, nc] contiguous: INCLUSIVE running sum of the stream
@@ -153,8 +153,8 @@ int cg_scan_lengths(const int32_t *lengths, int64_t n, int64_t *offsets,
 /* decode_function_gpu + do_dequantize + the final cast and layout (decoder.py:
  * 77-112, 24-34, 159-173) for every chunk at once.
  * cdf, maxima, offsets, payload: as written by cg_encode_kv (maxima in max_dt);
- *             payload_bytes < 4 GiB (decode longer caches in pieces); whole aligned 32-bit
- *             words of the payload are loaded, see cg_decode_fast_prefsum
+ *             whole aligned 32-bit words of the payload are loaded, see
+ *             cg_decode_fast_prefsum
  * out         device fp16/bf16 KV cache (out_dt, strides (ol, okv, ot, oh, 1)), written */
 int cg_decode_kv(const int16_t *cdf, int max_bins, const void *maxima, int max_dt,
                  const int64_t *offsets, const uint8_t *payload, int64_t payload_bytes,

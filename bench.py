@@ -32,6 +32,17 @@ WORKLOADS = {
     "config2_small": (32, 1024, 8, 128, 256, "mistralai/Mistral-7B-Instruct-v0.2", 1236),
     "config3": (32, 16384, 32, 128, 256, "mistralai/Mistral-7B-Instruct-v0.2", 1237),
     "config4": (80, 32768, 8, 128, 1500, "Yukang/LongAlpaca-70B-16k", 1238),
+    "config5": (32, 4096, 8, 128, 256, "levels", 1239),
+}
+
+# config 5: four quantization levels over the 32-layer tiers (first 10 / next 10 / rest for K,
+# first 2 / rest for V): A = 8 bins everywhere, B = reference QUANT_LEVEL 1, C = reference
+# QUANT_LEVEL 2, D = 64/32/32 and 64/32 (wider than the reference's tables allow).
+CONFIG5_LEVELS = {
+    "A": ((8, 8, 8), (8, 8)),
+    "B": ((16, 16, 12), (16, 12)),
+    "C": ((32, 16, 16), (32, 16)),
+    "D": ((64, 32, 32), (64, 32)),
 }
 
 
@@ -44,6 +55,58 @@ def bins_for(name, model, layers):
     os.environ.setdefault("QUANT_LEVEL", "2")
     cfg = B.CacheGenConfig.from_model_name(model)
     return B.make_key_bins(cfg), B.make_value_bins(cfg)
+
+
+def run_levels(args):
+    """config 5: the same cache encoded at four levels; prints one JSON line with a row per level."""
+    import torch
+    from cachegen_amd import codec
+    from cachegen_amd.kvgen import make_kv
+    from cachegen_amd.serde import cachegen_basics as B
+    L, T, H, D, chunk, _, seed = WORKLOADS["config5"]
+    dev = torch.device("cuda:0")
+    rho = [0.5 if l % 2 == 0 else 0.95 for l in range(L)]      # even layers rho 0.5, odd 0.95
+    kv = make_kv(L, T, H, D, seed=seed, rho=rho, device=dev)
+    C = H * D
+    workspace = torch.empty(codec.encode_workspace_bytes(L, T, C, chunk), dtype=torch.uint8, device=dev)
+    out = torch.empty((L, 2, T, H, D), dtype=torch.float16, device=dev)
+    kv_bytes = kv.numel() * 2
+    rows = {}
+    t_all = 0.0
+    for name, (kt, vt) in CONFIG5_LEVELS.items():
+        cfg = B.CacheGenConfig.from_layer_tiers(L, [(10, kt[0]), (20, kt[1]), kt[2]], [(2, vt[0]), vt[1]])
+        kb, vb = B.make_key_bins(cfg).to(dev), B.make_value_bins(cfg).to(dev)
+        max_bins = int(max(kt + vt))
+        enc = codec.encode_kv(kv, kb, vb, chunk_tokens=chunk, max_bins=max_bins, workspace=workspace)
+        enc.check()
+        for _ in range(args.warmup):
+            codec.encode_kv(kv, kb, vb, chunk_tokens=chunk, max_bins=max_bins, workspace=workspace, out=enc)
+            codec.decode_encoded(enc, kb, vb, fmt="vllm", out=out)
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+        ev[0].record()
+        for _ in range(args.steps):
+            codec.encode_kv(kv, kb, vb, chunk_tokens=chunk, max_bins=max_bins, workspace=workspace, out=enc)
+        ev[1].record()
+        for _ in range(args.steps):
+            codec.decode_encoded(enc, kb, vb, fmt="vllm", out=out)
+        ev[2].record()
+        torch.cuda.synchronize()
+        e_ms, d_ms = ev[0].elapsed_time(ev[1]) / args.steps, ev[1].elapsed_time(ev[2]) / args.steps
+        t_all += e_ms + d_ms
+        payload = enc.total_bytes()
+        side = 2 * (max_bins + 1) * 2 * L * C * enc.num_chunks + 4 * enc.lengths.numel() + 2 * 2 * L * T
+        rows[name] = {"bins": {"key": kt, "value": vt}, "encode_GBps": round(kv_bytes / e_ms / 1e6, 2),
+                      "decode_GBps": round(kv_bytes / d_ms / 1e6, 2),
+                      "compression_ratio_payload": round(kv_bytes / payload, 3),
+                      "compression_ratio_total": round(kv_bytes / (payload + side), 3)}
+    print(json.dumps({
+        "metric": "KV encode & decode GB/s (fp16 input) + % HBM roofline + compression ratio",
+        "value": round(2 * 4 * kv_bytes / (t_all * 1e-3) / 1e9, 3), "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(t_all, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "u32", "data": "synthetic",
+        "config": {"workload": "config5: 32 layers x {K,V} x 4096 tokens x 8 heads x 128, fp16, table per 256 tokens, "
+                               "four quantization levels, AR(1) rho 0.5 (even layers) / 0.95 (odd layers), seed %d" % seed},
+        "levels": rows}))
 
 
 def algorithmic_bytes(L, T, C, lp, nchunks, nstreams, payload):
@@ -94,6 +157,10 @@ def main():
         print("bench.py: this codec runs on one GPU; --gpus must be 1 (the path shards by layer or by "
               "token chunk with no exchange, see DESIGN.md)", file=sys.stderr)
         sys.exit(2)
+
+    if args.workload == "config5":
+        run_levels(args)
+        return
 
     import torch
     from cachegen_amd import codec

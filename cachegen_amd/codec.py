@@ -214,3 +214,16 @@ def quantize_kv(kv, key_bins, value_bins, fmt="vllm"):
             kv.data_ptr(), _DT[kv.dtype], L, T, H, D, sl, skv, st, sh,
             key_bins.data_ptr(), value_bins.data_ptr(), sym.data_ptr(), maxima.data_ptr(), _stream()))
     return sym, maxima
+
+
+def encode_kv_levels(kv, levels, chunk_tokens=None, fmt="vllm", workspace=None):
+    """Encode the same KV cache at several quantization levels (the adaptive-streaming
+    use of the reference: src/utils.py:357-377 and run_adaptation.py:63-72 pre-encode every
+    chunk at QUANT_LEVEL 1..3).  `levels` is a list of (key_bins, value_bins); returns one
+    EncodedKV per level.  The workspace is shared, the results are independent."""
+    (L, T, H, D), _ = _kv_strides(kv, fmt)
+    S = int(chunk_tokens) if chunk_tokens else T
+    ws_bytes = encode_workspace_bytes(L, T, H * D, S)
+    if workspace is None or workspace.numel() < ws_bytes:
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=kv.device)
+    return [encode_kv(kv, kb, vb, chunk_tokens=S, fmt=fmt, workspace=workspace) for kb, vb in levels]

@@ -30,11 +30,11 @@ SIGNATURES = {
     "cg_decode_fast_prefsum": (_INT, [_P, _INT, _P, _I64, _P, _I64, _I64, _I64, _P, _I64, _I64, _I64, _P]),
     "cg_quantize_kv": (_INT, [_P, _INT, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _P, _P, _P, _P, _P]),
     "cg_encode_kv_workspace": (_SZ, [_I64, _I64, _I64, _I64]),
-    "cg_encode_kv": (_INT, [_P, _INT, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _P, _P, _INT, _I64,
+    "cg_encode_kv": (_INT, [_P, _INT, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _P, _P, _INT, _I64, _INT,
                             _P, _P, _P, _P, _P, _I64, _P, _P, _SZ, _P]),
     "cg_scan_workspace": (_SZ, [_I64]),
     "cg_scan_lengths": (_INT, [_P, _I64, _P, _P, _SZ, _P]),
-    "cg_decode_kv": (_INT, [_P, _INT, _P, _INT, _P, _P, _I64, _P, _P, _I64, _I64, _I64, _I64, _I64,
+    "cg_decode_kv": (_INT, [_P, _INT, _P, _INT, _P, _P, _I64, _P, _P, _I64, _I64, _I64, _I64, _I64, _INT,
                             _P, _INT, _I64, _I64, _I64, _I64, _P]),
 }
 

@@ -55,6 +55,7 @@ class EncodedKV:
     head_size: int
     chunk_tokens: int
     max_bins: int
+    delta_group: int = 0       # > 0: delta-against-anchor groups (not part of the reference codec)
 
     @property
     def num_chunks(self):
@@ -106,11 +107,13 @@ def encode_workspace_bytes(num_layers, num_tokens, num_channels, chunk_tokens):
 
 
 def encode_kv(kv, key_bins, value_bins, chunk_tokens=None, fmt="vllm", max_bins=None,
-              workspace=None, out: Optional[EncodedKV] = None):
+              workspace=None, out: Optional[EncodedKV] = None, delta_group=0):
     """kv: fp16/bf16 GPU tensor [L,2,T,H,D] (fmt "vllm") or [L,2,H,T,D] ("huggingface").
     key_bins / value_bins: float32 GPU tensors [L].  chunk_tokens: tokens per table
     (default: all T, i.e. one `to_bytes` call).  `workspace` (uint8, GPU) and `out`
-    (a previous result of the same geometry) let a caller reuse memory."""
+    (a previous result of the same geometry) let a caller reuse memory.  delta_group > 0
+    switches on delta-against-anchor quantization in token groups of that size (an extension:
+    the reference codec has none); decode with the same value."""
     if not kv.is_cuda:
         raise RuntimeError("KV tensor should be on GPU")
     if kv.dtype not in _DT:
@@ -140,11 +143,12 @@ def encode_kv(kv, key_bins, value_bins, chunk_tokens=None, fmt="vllm", max_bins=
             offsets=torch.empty(nstreams + 1, dtype=torch.int64, device=dev),
             payload=torch.empty(nstreams * MAX_TOKENS_PER_STREAM, dtype=torch.uint8, device=dev),
             status=torch.empty(1, dtype=torch.int32, device=dev),
-            num_layers=L, num_tokens=T, num_heads=H, head_size=D, chunk_tokens=S, max_bins=max_bins)
+            num_layers=L, num_tokens=T, num_heads=H, head_size=D, chunk_tokens=S, max_bins=max_bins,
+            delta_group=int(delta_group))
     with torch.cuda.device(dev):
         _lib.check(lib.cg_encode_kv(
             kv.data_ptr(), _DT[kv.dtype], L, T, H, D, sl, skv, st, sh,
-            key_bins.data_ptr(), value_bins.data_ptr(), max_bins, S,
+            key_bins.data_ptr(), value_bins.data_ptr(), max_bins, S, int(delta_group),
             out.cdf.data_ptr(), out.maxima.data_ptr(), out.lengths.data_ptr(), out.offsets.data_ptr(),
             out.payload.data_ptr(), out.payload.numel(), out.status.data_ptr(),
             workspace.data_ptr(), workspace.numel(), _stream()))
@@ -165,7 +169,7 @@ def scan_lengths(lengths):
 
 
 def decode_kv(cdf, maxima, offsets, payload, key_bins, value_bins, num_layers, num_tokens,
-              num_heads, head_size, chunk_tokens, fmt="vllm", out_dtype=None, out=None):
+              num_heads, head_size, chunk_tokens, fmt="vllm", out_dtype=None, out=None, delta_group=0):
     """Inverse of `encode_kv`: returns the dequantized KV tensor, [L,2,T,H,D] for fmt "vllm"
     (default dtype bfloat16) or [L,2,H,T,D] for "huggingface" (default float16), as
     cachegen_decoder.py:169-173 does."""
@@ -189,7 +193,7 @@ def decode_kv(cdf, maxima, offsets, payload, key_bins, value_bins, num_layers, n
         _lib.check(_lib.lib().cg_decode_kv(
             cdf.data_ptr(), cdf.shape[-1] - 1, maxima.data_ptr(), _DT[maxima.dtype],
             offsets.data_ptr(), payload.data_ptr(), payload.numel(),
-            key_bins.data_ptr(), value_bins.data_ptr(), L, T, H, D, int(chunk_tokens),
+            key_bins.data_ptr(), value_bins.data_ptr(), L, T, H, D, int(chunk_tokens), int(delta_group),
             out.data_ptr(), _DT[out.dtype], ol, okv, ot, oh, _stream()))
     return out
 
@@ -197,7 +201,7 @@ def decode_kv(cdf, maxima, offsets, payload, key_bins, value_bins, num_layers, n
 def decode_encoded(enc: EncodedKV, key_bins, value_bins, fmt="vllm", out_dtype=None, out=None):
     return decode_kv(enc.cdf, enc.maxima, enc.offsets, enc.payload, key_bins, value_bins,
                      enc.num_layers, enc.num_tokens, enc.num_heads, enc.head_size,
-                     enc.chunk_tokens, fmt=fmt, out_dtype=out_dtype, out=out)
+                     enc.chunk_tokens, fmt=fmt, out_dtype=out_dtype, out=out, delta_group=enc.delta_group)
 
 
 def quantize_kv(kv, key_bins, value_bins, fmt="vllm"):

@@ -283,6 +283,7 @@ struct PackedQuantArgs {
     uint16_t *maxima;       // [2L, T]
     int32_t nunits;         // C / 8
     int64_t nsub;
+    int32_t delta_group;    // > 0: tokens of a sub-chunk in groups of this many, see below
     TokenGeom g;
 };
 
@@ -362,6 +363,103 @@ __global__ __launch_bounds__(256) void quantize_pack_kernel(PackedQuantArgs a)
             uint4 *dst = reinterpret_cast<uint4 *>(out + (int64_t)u * 8);
             dst[0] = make_uint4(words[0], words[1], words[2], words[3]);
             dst[1] = make_uint4(words[4], words[5], words[6], words[7]);
+        }
+    }
+}
+
+// Delta-against-anchor variant (no counterpart in the reference, off by default).  Inside
+// every sub-chunk the tokens form groups of `delta_group`; the first token of a group is its
+// anchor and is quantized as above, every other row is replaced by d = x - x_anchor
+// (float32) before the same quantization, with the row maximum of |d| rounded to the 16-bit
+// input format and symbols clamped to the table.  The decoder adds the reconstructed anchor
+// back.  Rows are handled one after the other so that registers hold one row, its anchor
+// and the packed result.
+template <int DT, bool HEADS_CONTIGUOUS, int NU>
+__global__ __launch_bounds__(256) void quantize_pack_delta_kernel(PackedQuantArgs a)
+{
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    int64_t b = blockIdx.x;
+    const int tq = (int)(b & 15) * 4 + wave;
+    b >>= 4;
+    const int64_t sub = b % a.nsub;
+    const int64_t row = b / a.nsub;
+    int64_t chunk, t0;
+    int n;
+    sub_range(a.g, sub, chunk, t0, n);
+    const int tt0 = tq * 4;
+    if (tt0 >= n) return;
+    const int nvalid = (n - tt0) < 4 ? (n - tt0) : 4;
+    const int64_t kvi = row / a.L, l = row - kvi * a.L;
+    const float bins = (kvi ? a.value_bins : a.key_bins)[l];
+    const float maxq = floorf(bins * 0.5f) - 1.0f;
+    const uint16_t *base = a.kv + l * a.sl + kvi * a.skv + t0 * a.st;     // token 0 of the sub-chunk
+
+    uint32_t words[NU][8];
+#pragma unroll
+    for (int i = 0; i < NU; ++i)
+#pragma unroll
+        for (int k = 0; k < 8; ++k) words[i][k] = 0;
+
+    for (int j = 0; j < nvalid; ++j) {
+        const int tt = tt0 + j;
+        const int ta = tt - tt % a.delta_group;          // the group's anchor
+        const bool is_anchor = ta == tt;
+        uint4 x[NU], xa[NU];
+        float m = 0.0f;
+#pragma unroll
+        for (int i = 0; i < NU; ++i) {
+            x[i] = make_uint4(0, 0, 0, 0);
+            xa[i] = make_uint4(0, 0, 0, 0);
+            const int u = lane + 64 * i;
+            if (u < a.nunits) {
+                const int e = u * 8;
+                int64_t off;
+                if (HEADS_CONTIGUOUS) off = e;
+                else { const int h = e / a.D; off = (int64_t)h * a.sh + (e - h * a.D); }
+                x[i] = *reinterpret_cast<const uint4 *>(base + tt * a.st + off);
+                if (!is_anchor) xa[i] = *reinterpret_cast<const uint4 *>(base + ta * a.st + off);
+                const uint32_t xs[4] = {x[i].x, x[i].y, x[i].z, x[i].w};
+                const uint32_t as[4] = {xa[i].x, xa[i].y, xa[i].z, xa[i].w};
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    const float v = load16f<DT>((k & 1) ? xs[k >> 1] >> 16 : xs[k >> 1] & 0xFFFFu);
+                    const float va = is_anchor ? 0.0f : load16f<DT>((k & 1) ? as[k >> 1] >> 16 : as[k >> 1] & 0xFFFFu);
+                    m = fmaxf(m, fabsf(__fsub_rn(v, va)));
+                }
+            }
+        }
+        m = __uint_as_float(wave_max_u32(__float_as_uint(m)));   // non-negative floats order as integers
+        uint32_t m16 = store16f<DT>(m);
+        const uint32_t inf16 = DT == CG_DT_BF16 ? 0x7F80u : 0x7C00u;
+        if (m16 >= inf16) m16 = inf16 - 1;                        // keep the stored maximum finite
+        if (lane == 0) a.maxima[row * a.g.T + t0 + tt] = (uint16_t)m16;
+        const float factor = __fdiv_rn(maxq, load16f<DT>(m16));
+        const float top = __fadd_rn(maxq, maxq);
+#pragma unroll
+        for (int i = 0; i < NU; ++i) {
+            const uint32_t xs[4] = {x[i].x, x[i].y, x[i].z, x[i].w};
+            const uint32_t as[4] = {xa[i].x, xa[i].y, xa[i].z, xa[i].w};
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const float v = load16f<DT>((k & 1) ? xs[k >> 1] >> 16 : xs[k >> 1] & 0xFFFFu);
+                const float va = is_anchor ? 0.0f : load16f<DT>((k & 1) ? as[k >> 1] >> 16 : as[k >> 1] & 0xFFFFu);
+                const float d = __fsub_rn(v, va);
+                const float sv = __fadd_rn(__fmul_rn(d, factor), maxq);
+                const float r = fminf(fmaxf(__builtin_rintf(sv), 0.0f), top);    // NaN -> 0, clamp to the table
+                words[i][k] |= ((uint32_t)(int)r & 0xFFu) << (8 * j);
+            }
+        }
+    }
+
+    const int64_t C = (int64_t)a.nunits * 8;
+    uint32_t *out = a.sym4 + ((row * a.nsub + sub) * kWordsPerSub + tq) * C;
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {
+        const int u = lane + 64 * i;
+        if (u < a.nunits) {
+            uint4 *dst = reinterpret_cast<uint4 *>(out + (int64_t)u * 8);
+            dst[0] = make_uint4(words[i][0], words[i][1], words[i][2], words[i][3]);
+            dst[1] = make_uint4(words[i][4], words[i][5], words[i][6], words[i][7]);
         }
     }
 }
@@ -931,6 +1029,7 @@ struct DecodeArgs {
     int32_t D;
     const uint16_t *maxima;     // [2, L, T]
     int32_t max_dt;
+    int32_t delta_group;        // > 0: rows that are not the first of their group hold deltas
     const float *key_bins, *value_bins;
     StreamGrid sg;
 };
@@ -999,6 +1098,8 @@ __global__ __launch_bounds__(BS) void decode_streams_kernel(DecodeArgs a)
     lds_f32 *const lutp = (lds_f32 *)lut;
     lds_f32 *rmp = (lds_f32 *)rowmax;
 
+    float anchor = 0.0f;               // reconstructed anchor row value (delta mode)
+    int phase = 0;                     // position of the token inside its group (delta mode)
     for (int i0 = 0; i0 < id.n; i0 += 4, rmp += 4) {
         // the maxima of the next four token rows (the array is padded to a multiple of four)
         float rm[4] = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -1068,7 +1169,12 @@ __global__ __launch_bounds__(BS) void decode_streams_kernel(DecodeArgs a)
                 osym[(int64_t)i * a.o1] = (uint8_t)(sym4 >> 2);
             } else {
                 const float q = *(lds_f32 *)((lds_char *)lutp + sym4);
-                const float v = __fmul_rn(q, rm[j]);
+                float v = __fmul_rn(q, rm[j]);
+                if (a.delta_group > 0) {                 // uniform over the block
+                    if (phase == 0) anchor = v;
+                    else v = __fadd_rn(v, anchor);
+                    phase = phase + 1 == a.delta_group ? 0 : phase + 1;
+                }
                 *okv = (uint16_t)(OUT == OUT_BF16 ? store16f<CG_DT_BF16>(v) : store16f<CG_DT_F16>(v));
                 okv += a.ot;
             }
@@ -1359,6 +1465,12 @@ template <int DT, bool HC>
 void launch_quantize_pack_nu(const PackedQuantArgs &a, int64_t nblocks, hipStream_t stream)
 {
     const dim3 grid((unsigned)nblocks), block(256);
+    if (a.delta_group > 0) {
+        if (a.nunits <= 128) quantize_pack_delta_kernel<DT, HC, 2><<<grid, block, 0, stream>>>(a);
+        else if (a.nunits <= 256) quantize_pack_delta_kernel<DT, HC, 4><<<grid, block, 0, stream>>>(a);
+        else quantize_pack_delta_kernel<DT, HC, 8><<<grid, block, 0, stream>>>(a);
+        return;
+    }
     if (a.nunits <= 128) quantize_pack_kernel<DT, HC, 2><<<grid, block, 0, stream>>>(a);
     else if (a.nunits <= 256) quantize_pack_kernel<DT, HC, 4><<<grid, block, 0, stream>>>(a);
     else quantize_pack_kernel<DT, HC, 8><<<grid, block, 0, stream>>>(a);
@@ -1367,7 +1479,7 @@ void launch_quantize_pack_nu(const PackedQuantArgs &a, int64_t nblocks, hipStrea
 int launch_quantize_pack(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D,
                          int64_t sl, int64_t skv, int64_t st, int64_t sh, const float *key_bins,
                          const float *value_bins, uint32_t *sym4, void *maxima, int64_t nsub,
-                         int64_t S, hipStream_t stream)
+                         int64_t S, int delta_group, hipStream_t stream)
 {
     PackedQuantArgs a;
     a.kv = static_cast<const uint16_t *>(kv);
@@ -1383,6 +1495,7 @@ int launch_quantize_pack(const void *kv, int kv_dt, int64_t L, int64_t T, int64_
     a.maxima = static_cast<uint16_t *>(maxima);
     a.nunits = (int32_t)(H * D / 8);
     a.nsub = nsub;
+    a.delta_group = delta_group;
     a.g.T = T;
     a.g.S = S;
     a.g.nsc = (int32_t)ceil_div(S, kSub);
@@ -1442,7 +1555,7 @@ void launch_decode_kv_log2(const DecodeArgs &a, dim3 grid, size_t shmem, hipStre
 extern "C" {
 
 const char *cg_last_error(void) { return g_error; }
-int cg_abi_version(void) { return 1; }
+int cg_abi_version(void) { return 2; }
 
 int64_t cg_num_chunks(int64_t T, int64_t chunk_tokens)
 {
@@ -1590,9 +1703,9 @@ size_t cg_encode_kv_workspace(int64_t L, int64_t T, int64_t C, int64_t chunk_tok
 
 int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D, int64_t sl,
                  int64_t skv, int64_t st, int64_t sh, const float *key_bins, const float *value_bins,
-                 int max_bins, int64_t chunk_tokens, int16_t *cdf, void *maxima, int32_t *lengths,
-                 int64_t *offsets, uint8_t *payload, int64_t payload_cap, int32_t *status,
-                 void *workspace, size_t workspace_bytes, void *stream)
+                 int max_bins, int64_t chunk_tokens, int delta_group, int16_t *cdf, void *maxima,
+                 int32_t *lengths, int64_t *offsets, uint8_t *payload, int64_t payload_cap,
+                 int32_t *status, void *workspace, size_t workspace_bytes, void *stream)
 {
     if (!kv || !key_bins || !value_bins || !cdf || !maxima || !lengths || !offsets || !payload || !status || !workspace)
         return fail(CG_ERR_ARG, "encode_kv: null pointer");
@@ -1601,6 +1714,7 @@ int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int
     if (chunk_tokens <= 0) return fail(CG_ERR_ARG, "encode_kv: chunk_tokens must be positive");
     if (chunk_tokens > 65535) return fail(CG_ERR_ARG, "encode_kv: at most 65535 tokens per chunk (16-bit counters)");
     if (int rc = check_lp(max_bins + 1, "encode_kv")) return rc;
+    if (delta_group < 0 || delta_group > kSub) return fail(CG_ERR_ARG, "encode_kv: delta_group must be in [0, %d]", kSub);
     const int64_t C = H * D, rows = 2 * L;
     const int64_t nsub = cg_num_subchunks(T, chunk_tokens);
     const int64_t nstreams = nsub * rows * C;
@@ -1635,11 +1749,13 @@ int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int
     const dim3 grid((unsigned)nblocks), blk(block);
 
     const bool packed = kv_vectorizable(kv, D, C, sl, skv, st, sh) && C % 8 == 0;
+    if (delta_group > 0 && !packed)
+        return fail(CG_ERR_ARG, "encode_kv: delta groups need head sizes and strides that are multiples of 8 and a 16-byte aligned tensor");
     if (packed) {
         // four tokens per word, read by one lane per channel
         uint32_t *sym4 = reinterpret_cast<uint32_t *>(symbols);
         if (int rc = launch_quantize_pack(kv, kv_dt, L, T, H, D, sl, skv, st, sh, key_bins, value_bins, sym4,
-                                          maxima, nsub, chunk_tokens, s)) return rc;
+                                          maxima, nsub, chunk_tokens, delta_group, s)) return rc;
         a.sym4 = sym4;
         if (chunk_tokens <= kSub) {
             // one sub-chunk per chunk: the encoder builds the tables itself
@@ -1672,8 +1788,8 @@ int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int
 int cg_decode_kv(const int16_t *cdf, int max_bins, const void *maxima, int max_dt, const int64_t *offsets,
                  const uint8_t *payload, int64_t payload_bytes, const float *key_bins,
                  const float *value_bins, int64_t L, int64_t T, int64_t H, int64_t D,
-                 int64_t chunk_tokens, void *out, int out_dt, int64_t ol, int64_t okv, int64_t ot,
-                 int64_t oh, void *stream)
+                 int64_t chunk_tokens, int delta_group, void *out, int out_dt, int64_t ol, int64_t okv,
+                 int64_t ot, int64_t oh, void *stream)
 {
     if (!cdf || !maxima || !offsets || !key_bins || !value_bins || !out || !payload)
         return fail(CG_ERR_ARG, "decode_kv: null pointer");
@@ -1681,6 +1797,7 @@ int cg_decode_kv(const int16_t *cdf, int max_bins, const void *maxima, int max_d
     if (int rc = check_dt(out_dt, "decode_kv")) return rc;
     if (L <= 0 || T <= 0 || H <= 0 || D <= 0 || chunk_tokens <= 0) return fail(CG_ERR_ARG, "decode_kv: empty input");
     if (int rc = check_lp(max_bins + 1, "decode_kv")) return rc;
+    if (delta_group < 0 || delta_group > kSub) return fail(CG_ERR_ARG, "decode_kv: delta_group must be in [0, %d]", kSub);
     const int64_t C = H * D, rows = 2 * L;
     if (D > INT_MAX) return fail(CG_ERR_ARG, "decode_kv: head size too large");
     const int64_t nsub = cg_num_subchunks(T, chunk_tokens);
@@ -1700,6 +1817,7 @@ int cg_decode_kv(const int16_t *cdf, int max_bins, const void *maxima, int max_d
     a.D = (int32_t)D;
     a.maxima = static_cast<const uint16_t *>(maxima);
     a.max_dt = max_dt;
+    a.delta_group = delta_group;
     a.key_bins = key_bins;
     a.value_bins = value_bins;
     int64_t nblocks;

@@ -134,11 +134,17 @@ size_t cg_encode_kv_workspace(int64_t L, int64_t T, int64_t C, int64_t chunk_tok
  *             always enough.
  * status      device int32 [1], written: 0, or 1 if a stream exceeded 256 bytes
  *             (the reference overruns its buffer there; here the stream is cut).
- * workspace   device scratch of cg_encode_kv_workspace(...) bytes, 256-aligned */
+ * workspace   device scratch of cg_encode_kv_workspace(...) bytes, 256-aligned
+ * delta_group 0 for the reference's codec.  > 0 (no counterpart in the reference): inside
+ *             every sub-chunk, tokens form groups of this many; the first row of a group
+ *             (the anchor) is quantized as is, every other row as its float32 difference
+ *             from the anchor row, with the row maximum of the differences rounded to the
+ *             16-bit format; cg_decode_kv with the same value adds the reconstructed
+ *             anchor back. */
 int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D,
                  int64_t sl, int64_t skv, int64_t st, int64_t sh,
                  const float *key_bins, const float *value_bins, int max_bins,
-                 int64_t chunk_tokens,
+                 int64_t chunk_tokens, int delta_group,
                  int16_t *cdf, void *maxima, int32_t *lengths, int64_t *offsets,
                  uint8_t *payload, int64_t payload_cap, int32_t *status,
                  void *workspace, size_t workspace_bytes, void *stream);
@@ -160,6 +166,7 @@ int cg_decode_kv(const int16_t *cdf, int max_bins, const void *maxima, int max_d
                  const int64_t *offsets, const uint8_t *payload, int64_t payload_bytes,
                  const float *key_bins, const float *value_bins,
                  int64_t L, int64_t T, int64_t H, int64_t D, int64_t chunk_tokens,
+                 int delta_group,
                  void *out, int out_dt, int64_t ol, int64_t okv, int64_t ot, int64_t oh,
                  void *stream);
 

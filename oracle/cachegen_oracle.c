@@ -174,6 +174,83 @@ void cgo_dequantize(const uint8_t *sym, int64_t nl, int64_t nt, int64_t nc,
 }
 
 /* ------------------------------------------------------------------------ */
+/* Delta-against-anchor variant of the two functions above.  It has NO         */
+/* counterpart in the reference (its snapshot holds no anchor/delta code), so  */
+/* there is no parity target: this is the definition the HIP path is checked   */
+/* against, pinned by a hand known-answer, by "group = 0 or 1 gives the plain  */
+/* functions" and by the reconstruction bound.  Tokens are taken in sub-chunks */
+/* of 256; inside a sub-chunk they form groups of `group`; the first row of a  */
+/* group (the anchor) is quantized as is, every other row as d = x - x_anchor  */
+/* in float32, with max|d| rounded to the 16-bit format (kept finite) and the  */
+/* symbols clamped to [0, 2*MAX].  Dequantization adds the anchor's float32    */
+/* reconstruction back before the 16-bit cast.                                 */
+/* ------------------------------------------------------------------------ */
+void cgo_quantize_delta(const uint16_t *x, int dt, int64_t nl, int64_t nt, int64_t nc,
+                        int64_t sl, int64_t st, const float *bins, int group,
+                        uint8_t *sym, uint16_t *max_out)
+{
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int64_t l = 0; l < nl; l++) {
+        for (int64_t t = 0; t < nt; t++) {
+            const int64_t w = t % 256;
+            const int64_t ta = t - (w % group);
+            const uint16_t *row = x + l * sl + t * st;
+            const uint16_t *arow = x + l * sl + ta * st;
+            const float maxq = floorf(bins[l] / 2.0f) - 1.0f;
+            float m = 0.0f;
+            for (int64_t c = 0; c < nc; c++) {
+                float v = load16(row + c, dt);
+                float va = (ta == t) ? 0.0f : load16(arow + c, dt);
+                float d = fabsf(v - va);
+                if (d > m) m = d;               /* NaN differences are ignored, like fmaxf */
+            }
+            uint16_t m16 = store16(m, dt);
+            const uint16_t inf16 = dt == CGO_DT_BF16 ? 0x7F80u : 0x7C00u;
+            if (m16 >= inf16) m16 = (uint16_t)(inf16 - 1);
+            max_out[l * nt + t] = m16;
+            const float factor = maxq / load16(&m16, dt);
+            const float top = maxq + maxq;
+            uint8_t *out = sym + (l * nt + t) * nc;
+            for (int64_t c = 0; c < nc; c++) {
+                float v = load16(row + c, dt);
+                float va = (ta == t) ? 0.0f : load16(arow + c, dt);
+                float d = v - va;
+                float p = d * factor;
+                float s = p + maxq;
+                float r = rintf(s);
+                if (r != r) r = 0.0f;
+                if (r < 0.0f) r = 0.0f;
+                if (r > top) r = top;
+                out[c] = (uint8_t)(int)r;
+            }
+        }
+    }
+}
+
+void cgo_dequantize_delta(const uint8_t *sym, int64_t nl, int64_t nt, int64_t nc,
+                          const float *bins, const uint16_t *maxima, int max_dt, int group,
+                          uint16_t *out, int64_t ol, int64_t ot, int out_dt)
+{
+#pragma omp parallel for schedule(static)
+    for (int64_t l = 0; l < nl; l++) {
+        const float cq = floorf(bins[l] / 2.0f) - 1.0f;
+        for (int64_t c = 0; c < nc; c++) {
+            float anchor = 0.0f;
+            for (int64_t t = 0; t < nt; t++) {
+                const float m = load16(maxima + l * nt + t, max_dt);
+                float v = (float)sym[(l * nt + t) * nc + c];
+                v = v - cq;
+                v = v / cq;
+                v = v * m;
+                if ((t % 256) % group == 0) anchor = v;
+                else v = v + anchor;
+                out[l * ol + t * ot + c] = store16(v, out_dt);
+            }
+        }
+    }
+}
+
+/* ------------------------------------------------------------------------ */
 /* CDF: calculate_cdf_kernel + normalize_cdf_value, cal_cdf.cu:11-14,29-49.  */
 /* Per (layer, channel): 16-bit counters hist[sym+1]++ over all tokens, an   */
 /* inclusive running sum, then                                               */

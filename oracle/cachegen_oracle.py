@@ -102,6 +102,30 @@ def dequantize(sym, bins, maxima, max_dt=DT_F16, out_dt=DT_F16):
     return out
 
 
+def quantize_delta(x_bits, bins, group, dt=DT_F16):
+    """Delta-against-anchor quantization (no counterpart in the reference; see the C file)."""
+    nl, nt, nc = x_bits.shape
+    s = _estrides(x_bits)
+    bins = np.ascontiguousarray(bins, dtype=np.float32)
+    sym = np.empty((nl, nt, nc), dtype=np.uint8)
+    mx = np.empty((nl, nt), dtype=np.uint16)
+    lib().cgo_quantize_delta(_p(x_bits), ctypes.c_int(dt), _i64(nl), _i64(nt), _i64(nc), _i64(s[0]),
+                             _i64(s[1]), _p(bins), ctypes.c_int(group), _p(sym), _p(mx))
+    return sym, mx
+
+
+def dequantize_delta(sym, bins, maxima, group, max_dt=DT_F16, out_dt=DT_F16):
+    sym = np.ascontiguousarray(sym, dtype=np.uint8)
+    nl, nt, nc = sym.shape
+    bins = np.ascontiguousarray(bins, dtype=np.float32)
+    maxima = np.ascontiguousarray(maxima, dtype=np.uint16).reshape(nl, nt)
+    out = np.empty((nl, nt, nc), dtype=np.uint16)
+    lib().cgo_dequantize_delta(_p(sym), _i64(nl), _i64(nt), _i64(nc), _p(bins), _p(maxima),
+                               ctypes.c_int(max_dt), ctypes.c_int(group), _p(out), _i64(nt * nc),
+                               _i64(nc), ctypes.c_int(out_dt))
+    return out
+
+
 def calculate_cdf(sym, max_bins):
     """sym uint8/int8 [nl, nt, nc] (any strides) -> uint16 [nl, nc, max_bins + 1]."""
     sym = sym.view(np.uint8)
@@ -194,7 +218,7 @@ def decode_fast_new(cdf, padded, lengths, nt, out=None):
     return out
 
 
-def encode_function(kv_bits, key_bins, value_bins, dt=DT_F16):
+def encode_function(kv_bits, key_bins, value_bins, dt=DT_F16, delta_group=0):
     """One `to_bytes` call (encoder.py:247-301) on kv_bits uint16 [L, 2, T, C].
 
     Returns a dict with the fields of CacheGenGPUEncoderOutput as numpy arrays:
@@ -205,8 +229,12 @@ def encode_function(kv_bits, key_bins, value_bins, dt=DT_F16):
     assert two == 2
     key_bins = np.asarray(key_bins, dtype=np.float32)
     value_bins = np.asarray(value_bins, dtype=np.float32)
-    sym_k, max_k = quantize(kv_bits[:, 0], key_bins, dt)
-    sym_v, max_v = quantize(kv_bits[:, 1], value_bins, dt)
+    if delta_group > 0:
+        sym_k, max_k = quantize_delta(kv_bits[:, 0], key_bins, delta_group, dt)
+        sym_v, max_v = quantize_delta(kv_bits[:, 1], value_bins, delta_group, dt)
+    else:
+        sym_k, max_k = quantize(kv_bits[:, 0], key_bins, dt)
+        sym_v, max_v = quantize(kv_bits[:, 1], value_bins, dt)
     sym = np.concatenate([sym_k, sym_v], axis=0)
     cdf = np.concatenate([calculate_cdf(sym_k, int(key_bins.max())),
                           calculate_cdf(sym_v, int(value_bins.max()))], axis=0)
@@ -221,7 +249,7 @@ def encode_function(kv_bits, key_bins, value_bins, dt=DT_F16):
                 data_chunks=chunks, symbols=sym)
 
 
-def decode_function(enc, key_bins, value_bins, max_dt=DT_F16, out_dt=DT_F16):
+def decode_function(enc, key_bins, value_bins, max_dt=DT_F16, out_dt=DT_F16, delta_group=0):
     """One `from_bytes` call (decoder.py:144-173) up to the [L, 2, T, C] blob.
 
     Returns (symbols uint8 [2L, T, C], kv_bits uint16 [L, 2, T, C])."""
@@ -235,6 +263,10 @@ def decode_function(enc, key_bins, value_bins, max_dt=DT_F16, out_dt=DT_F16):
         prefix = lengths.astype(np.int64).ravel().cumsum().reshape(lengths.shape)
         decode_fast_prefsum(cdf, data, prefix, n, sym[:, start:start + n, :])
         start += n
-    k = dequantize(sym[:nl], key_bins, enc["max_tensors_key"], max_dt, out_dt)
-    v = dequantize(sym[nl:], value_bins, enc["max_tensors_value"], max_dt, out_dt)
+    if delta_group > 0:
+        k = dequantize_delta(sym[:nl], key_bins, enc["max_tensors_key"], delta_group, max_dt, out_dt)
+        v = dequantize_delta(sym[nl:], value_bins, enc["max_tensors_value"], delta_group, max_dt, out_dt)
+    else:
+        k = dequantize(sym[:nl], key_bins, enc["max_tensors_key"], max_dt, out_dt)
+        v = dequantize(sym[nl:], value_bins, enc["max_tensors_value"], max_dt, out_dt)
     return sym, np.stack([k, v], axis=1)

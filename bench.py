@@ -149,13 +149,13 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="config2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-sample-tokens", type=int, default=1024)
+    ap.add_argument("--cpu-sample-tokens", type=int, default=8192)
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one plain device copy of the KV tensor (calibrates rocprofv3 byte counters)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this codec runs on one GPU; --gpus must be 1 (the path shards by layer or by "
-              "token chunk with no exchange, see DESIGN.md)", file=sys.stderr)
+              "token chunk with no exchange)", file=sys.stderr)
         sys.exit(2)
 
     if args.workload == "config5":

@@ -117,18 +117,10 @@ __device__ __forceinline__ uint32_t store16f(float f)
 // int, which would turn a following >> into an arithmetic shift).
 __device__ __forceinline__ uint32_t mul24(uint32_t a, uint32_t b) { return (uint32_t)__umul24(a, b); }
 
-// floor(span * c / 2^16) for span = r + 1 (rh = r >> 16, rl = r & 0xffff) and a table
-// value c <= 0xffff, on the full-rate 24-bit multiplier: span*c = rh*c*2^16 + (rl+1)*c.
-// This is `(span * c) >> precision` of enc_new.cu:272-273 / dec_new.cu:280-281.
-__device__ __forceinline__ uint32_t scale16(uint32_t rh, uint32_t rl, uint32_t c)
-{
-    const uint32_t lowpart = mul24(rl, c) + c;
-    return mul24(rh, c) + (lowpart >> 16);
-}
-
-// The same product from the span itself (sh = span >> 16, sl = span & 0xffff), valid for
-// every span below 2^32 and every c up to and including 2^16 (where it returns the span):
-// span*c = sh*c*2^16 + sl*c.
+// floor(span * c / 2^16), the `(span * c) >> precision` of enc_new.cu:272-273 and
+// dec_new.cu:280-281, on the full-rate 24-bit multiplier from the span's halves
+// (sh = span >> 16, sl = span & 0xffff): span*c = sh*c*2^16 + sl*c.  Valid for every span
+// below 2^32 and every c up to and including 2^16 (where it returns the span).
 __device__ __forceinline__ uint32_t scale_span(uint32_t sh, uint32_t sl, uint32_t c)
 {
     return mul24(sh, c) + (mul24(sl, c) >> 16);

@@ -7,6 +7,7 @@ import torch
 from .. import codec, torchac_hip
 from ..config import LMCacheEngineConfig, LMCacheEngineMetadata
 from . import cachegen_basics as CGBasics
+from . import wire
 from .cachegen_basics import CacheGenConfig, CacheGenGPUBytestream, CacheGenGPUEncoderOutput
 from .serde import Deserializer
 
@@ -61,7 +62,9 @@ class CacheGenDeserializer(Deserializer):
         """Returns bfloat16 [num_layers, 2, num_tokens, num_heads, head_size] for fmt "vllm",
         float16 [num_layers, 2, num_heads, num_tokens, head_size] for "huggingface"
         (cachegen_decoder.py:144-173).  Decode, dequantization, cast and layout are one
-        kernel."""
+        kernel.  Blobs in the flat container of `wire` are recognised by their magic."""
+        if wire.is_flat(bs):
+            return self._from_flat(bs)
         encoder_output = CacheGenGPUEncoderOutput.from_bytes(bs)
         cdf = encoder_output.cdf.cuda()
         max_k = encoder_output.max_tensors_key.cuda()
@@ -79,3 +82,16 @@ class CacheGenDeserializer(Deserializer):
         return codec.decode_kv(cdf.unsqueeze(0), maxima, offsets, payload, self.key_bins,
                                self.value_bins, nlayers, ntokens, encoder_output.num_heads,
                                encoder_output.head_size, chunk_tokens=ntokens, fmt=self.fmt)
+
+    def _from_flat(self, bs) -> torch.Tensor:
+        h, cdf, maxima, lengths, payload = wire.unpack_to_device(bs, self.key_bins.device)
+        if h["num_layers"] != self.key_bins.numel():
+            raise ValueError("blob has %d layers, this deserializer's model %d"
+                             % (h["num_layers"], self.key_bins.numel()))
+        offsets = codec.scan_lengths(lengths)
+        total, shortest = torch.stack([offsets[-1], lengths.min().to(torch.int64)]).tolist()
+        if total != h["payload_bytes"] or shortest < 0:
+            raise ValueError("wire container: payload size is not the sum of the stream lengths")
+        return codec.decode_kv(cdf, maxima, offsets, payload, self.key_bins, self.value_bins,
+                               h["num_layers"], h["num_tokens"], h["num_heads"], h["head_size"],
+                               chunk_tokens=h["chunk_tokens"], fmt=self.fmt, delta_group=h["delta_group"])

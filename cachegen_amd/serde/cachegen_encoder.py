@@ -5,6 +5,7 @@ import torch
 from .. import codec, torchac_hip
 from ..config import LMCacheEngineConfig, LMCacheEngineMetadata
 from . import cachegen_basics as CGBasics
+from . import wire
 from .cachegen_basics import CacheGenConfig, CacheGenGPUBytestream, CacheGenGPUEncoderOutput
 from .serde import Serializer
 
@@ -49,7 +50,14 @@ def encode_function(kv: torch.Tensor, config: CacheGenConfig, key_bins: torch.Te
 
 
 class CacheGenSerializer(Serializer):
-    def __init__(self, config: LMCacheEngineConfig, metadata: LMCacheEngineMetadata):
+    def __init__(self, config: LMCacheEngineConfig, metadata: LMCacheEngineMetadata,
+                 wire_format: str = "pickle"):
+        """wire_format "pickle": the reference's container (cachegen_basics.py:110-122);
+        "flat": the versioned flat container of `wire`, which `CacheGenDeserializer` reads
+        as well."""
+        if wire_format not in ("pickle", "flat"):
+            raise ValueError(f"Invalid wire format: {wire_format}")
+        self.wire_format = wire_format
         self.cachegen_config = CacheGenConfig.from_model_name(metadata.model_name)
         self.chunk_size = config.chunk_size
         self.fmt = metadata.fmt
@@ -69,6 +77,9 @@ class CacheGenSerializer(Serializer):
         if self.fmt == "huggingface":
             tensor = tensor.permute(0, 1, 3, 2, 4)
         ntokens = tensor.shape[2]
+        if self.wire_format == "flat":
+            enc = codec.encode_kv(tensor.cuda(), self.key_bins, self.value_bins, chunk_tokens=ntokens)
+            return wire.pack_chunks(enc, per_chunk=False)[0]
         output = encode_function(tensor.cuda(), self.cachegen_config, self.key_bins,
                                  self.value_bins, ntokens)
         return output.to_bytes()

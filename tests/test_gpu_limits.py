@@ -1,0 +1,111 @@
+"""Limits and error reporting of the HIP path: streams cut at the buffer size, streams that
+outgrow 256 bytes, a payload buffer that is too small.  The reference has no defined
+behaviour for the last two (enc_new.cu:323-340 writes past its 256-byte slot); here they
+are reported through the status word and nothing is written out of bounds."""
+import dataclasses
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def _mods():
+    from cachegen_amd import codec, torchac_hip
+    return codec, torchac_hip
+
+
+@pytest.mark.parametrize("cap", [1, 7, 64, 130])
+def test_entry_point_cuts_streams_at_the_buffer_size(oracle, cap):
+    """Full length reported, `cap` bytes stored, nothing past the row touched: the oracle's
+    bit_sink does the same (it counts bytes it cannot store)."""
+    _, tac = _mods()
+    rng = np.random.default_rng(cap)
+    nl, nt, nc = 2, 256, 70
+    sym = rng.integers(0, 31, size=(nl, nt, nc), dtype=np.uint8)       # ~4.9 bits/symbol: ~157 bytes
+    cdf = oracle.calculate_cdf(sym, 32)
+    want_pad, want_len = oracle.encode_fast_new(cdf, sym, cap=cap)
+    assert want_len.max() > cap
+    guard = 5
+    big = torch.full((nl, nc, cap + guard), 0xEE, dtype=torch.uint8, device=DEV)
+    out = big[:, :, :cap]
+    lens = torch.zeros((nl, nc), dtype=torch.int32, device=DEV)
+    tac.encode_fast_new(torch.from_numpy(cdf.view(np.int16)).to(DEV),
+                        torch.from_numpy(sym).to(DEV).view(torch.int8), out, lens)
+    assert np.array_equal(lens.cpu().numpy(), want_len)
+    got = big.cpu().numpy()
+    stored = np.minimum(want_len, cap)
+    mask = np.arange(cap)[None, None, :] < stored[..., None]
+    assert np.array_equal(got[:, :, :cap][mask], want_pad[mask])
+    assert (got[:, :, cap:] == 0xEE).all()
+
+
+def _overflowing_kv(T, C=64):
+    """One layer; channel 1 carries the row maximum, channel 0 is -max on even tokens and
+    -max/3 on odd tokens of the first 256 tokens and +max elsewhere: with one table over
+    T = 65280 tokens the two symbols of the first sub-chunk have probability 128/65280
+    each, i.e. 9 bits per symbol and 288 bytes for that stream."""
+    kv = torch.zeros((1, 2, T, 1, C), dtype=torch.float16)
+    kv[..., 1] = 1.0
+    kv[..., 0] = 1.0
+    kv[:, :, 0:256:2, :, 0] = -1.0
+    kv[:, :, 1:256:2, :, 0] = -1.0 / 3.0
+    return kv
+
+
+def test_stream_longer_than_256_bytes_is_reported(oracle):
+    codec, _ = _mods()
+    T = 65280
+    kv = _overflowing_kv(T)
+    bins = torch.tensor([32.0])
+    enc = codec.encode_kv(kv.to(DEV), bins, bins, chunk_tokens=T)
+    with pytest.raises(RuntimeError, match="exceeded 256 bytes"):
+        enc.check()
+    lengths = enc.lengths.cpu().numpy()
+    # the oracle's coder on the same symbols gives the uncut length
+    flat = kv.reshape(1, 2, T, 64).contiguous().view(torch.int16).numpy().view(np.uint16)
+    want = oracle.encode_function(flat, bins.numpy(), bins.numpy())
+    assert np.array_equal(enc.cdf[0].cpu().numpy().view(np.uint16), want["cdf"])
+    data0, want_first, ntok = want["data_chunks"][0]
+    assert ntok == 256 and want_first[0, 0] > 256 and want_first[1, 0] > 256
+    assert np.array_equal(lengths[0], want_first)
+    # offsets advance by the stored (cut) length and every other stream is intact
+    offs = enc.offsets.cpu().numpy()
+    stored = np.minimum(lengths, 256)
+    assert np.array_equal(np.diff(offs), stored.ravel())
+    per_sub = lengths[0].size
+    got0 = enc.payload[:offs[per_sub]].cpu().numpy()
+    assert np.array_equal(got0, data0)                      # the oracle cuts at 256 bytes as well
+    # the last sub-chunk (all streams short) decodes to its symbols
+    last = lengths.shape[0] - 1
+    data_l, len_l, n_l = want["data_chunks"][last]
+    assert np.array_equal(enc.payload[offs[last * per_sub]:offs[(last + 1) * per_sub]].cpu().numpy(), data_l)
+    assert np.array_equal(lengths[last], len_l)
+
+
+def test_payload_buffer_too_small_is_reported():
+    codec, _ = _mods()
+    from cachegen_amd.kvgen import make_kv
+    kv = make_kv(2, 300, 4, 64, seed=5, device=DEV)
+    bins = torch.tensor([32.0, 16.0])
+    enc = codec.encode_kv(kv, bins, bins, chunk_tokens=256)
+    enc.check()
+    total = enc.total_bytes()
+    want = enc.payload[:total].cpu()
+
+    exact = dataclasses.replace(enc, payload=torch.full((total + 64,), 0xEE, dtype=torch.uint8, device=DEV)[:total],
+                                status=torch.zeros(1, dtype=torch.int32, device=DEV))
+    codec.encode_kv(kv, bins, bins, chunk_tokens=256, out=exact)
+    exact.check()
+    assert torch.equal(exact.payload.cpu(), want)
+
+    base = torch.full((total + 64,), 0xEE, dtype=torch.uint8, device=DEV)
+    small = dataclasses.replace(enc, payload=base[:total - 1],
+                                status=torch.zeros(1, dtype=torch.int32, device=DEV))
+    codec.encode_kv(kv, bins, bins, chunk_tokens=256, out=small)
+    with pytest.raises(RuntimeError, match="payload buffer too small"):
+        small.check()
+    assert (base[total - 1:] == 0xEE).all()                 # nothing written past the buffer

@@ -1,0 +1,159 @@
+"""The flat wire container (cachegen_amd/serde/wire.py): layout known answers and validation
+on the CPU, and on the GPU the equality of the device-assembled blobs with the host
+definition and of the decoded tensors with the pickle container's."""
+import pickle
+import struct
+
+import numpy as np
+import pytest
+import torch
+
+from cachegen_amd.serde import wire
+
+
+def _small_arrays(rng, L=1, T=300, H=1, D=2, S=300, lp=5):
+    C = H * D
+    nchunks = -(-T // S)
+    nsub = wire.geometry(L, T, H, D, S, lp - 1, 0)["nsub"][0]
+    cdf = rng.integers(0, 65536, size=(nchunks, 2 * L, C, lp), dtype=np.uint16)
+    maxima = rng.integers(0, 65536, size=(2, L, T), dtype=np.uint16)
+    lengths = rng.integers(1, 200, size=(nsub, 2 * L, C)).astype(np.int32)
+    payload = rng.integers(0, 256, size=int(lengths.sum()), dtype=np.uint8)
+    return cdf, maxima, lengths, payload
+
+
+def test_layout_known_answer():
+    """L=1, T=300, H=1, D=2, one table: sections at 64, 64+40->128, 128+1200->1344, 1344+32->1408."""
+    rng = np.random.default_rng(0)
+    cdf, maxima, lengths, payload = _small_arrays(rng)
+    assert cdf.nbytes == 40 and maxima.nbytes == 1200 and lengths.nbytes == 32
+    blob = wire.pack_host(cdf, maxima, lengths, payload, num_heads=1, head_size=2, chunk_tokens=300)
+    assert blob[:4] == b"CGKV"
+    assert struct.unpack_from("<HH", blob, 4) == (1, 0)
+    assert struct.unpack_from("<8I", blob, 8) == (1, 300, 1, 2, 300, 4, 0, 2)
+    assert struct.unpack_from("<Q", blob, 40) == (payload.size,)
+    assert blob[48:64] == bytes(16)
+    assert blob[64:104] == cdf.tobytes() and blob[104:128] == bytes(24)
+    assert blob[128:1328] == maxima.tobytes() and blob[1328:1344] == bytes(16)
+    assert blob[1344:1376] == lengths.tobytes()
+    assert blob[1408:1408 + payload.size] == payload.tobytes()
+    assert len(blob) == 1408 + (payload.size + 63) // 64 * 64
+    assert wire.is_flat(blob) and not wire.is_flat(pickle.dumps({"a": 1})) and not wire.is_flat(b"")
+
+
+@pytest.mark.parametrize("T,S", [(300, 300), (700, 256), (1500, 1500), (1501, 600)])
+def test_host_round_trip(T, S):
+    rng = np.random.default_rng(T)
+    cdf, maxima, lengths, payload = _small_arrays(rng, L=2, T=T, H=2, D=3, S=S, lp=17)
+    blob = wire.pack_host(cdf, maxima, lengths, payload, 2, 3, S, delta_group=4, bf16_maxima=True)
+    h, c2, m2, l2, p2 = wire.unpack_host(blob)
+    assert (h["num_layers"], h["num_tokens"], h["num_heads"], h["head_size"]) == (2, T, 2, 3)
+    assert (h["chunk_tokens"], h["max_bins"], h["delta_group"], h["bf16_maxima"]) == (S, 16, 4, True)
+    for a, b in ((cdf, c2), (maxima, m2), (lengths, l2), (payload, p2)):
+        assert a.dtype == b.dtype and np.array_equal(a, b)
+
+
+def test_sub_chunk_count_follows_the_chunking():
+    # 1501 tokens cut every 600: chunks of 600, 600, 301 tokens -> 3 + 3 + 2 sub-chunks
+    assert wire.geometry(1, 1501, 1, 1, 600, 4, 0)["nsub"][0] == 8
+    assert wire.geometry(1, 1501, 1, 1, 600, 4, 0)["nchunks"][0] == 3
+    assert wire.geometry(1, 256, 1, 1, 256, 4, 0)["nsub"][0] == 1
+
+
+def test_invalid_blobs_are_rejected():
+    rng = np.random.default_rng(3)
+    cdf, maxima, lengths, payload = _small_arrays(rng)
+    blob = wire.pack_host(cdf, maxima, lengths, payload, 1, 2, 300)
+    with pytest.raises(ValueError, match="bad magic"):
+        wire.read_header(b"XXXX" + blob[4:])
+    with pytest.raises(ValueError, match="version"):
+        wire.read_header(blob[:4] + struct.pack("<H", 9) + blob[6:])
+    with pytest.raises(ValueError, match="unknown flags"):
+        wire.read_header(blob[:6] + struct.pack("<H", 0x80) + blob[8:])
+    with pytest.raises(ValueError, match="geometry gives"):
+        wire.read_header(blob[:-64])
+    with pytest.raises(ValueError, match="shorter than its header"):
+        wire.read_header(blob[:10])
+    with pytest.raises(ValueError, match="sub-chunks recorded"):
+        wire.read_header(blob[:36] + struct.pack("<I", 3) + blob[40:])
+    bad = bytearray(blob)
+    bad[1344:1348] = struct.pack("<i", int(lengths.flat[0]) + 1)      # one length no longer matches
+    with pytest.raises(ValueError, match="sum of the stream lengths"):
+        wire.unpack_host(bytes(bad))
+    with pytest.raises(ValueError, match="sum of the stream lengths"):
+        wire.pack_host(cdf, maxima, lengths, payload[:-1], 1, 2, 300)
+    with pytest.raises(ValueError, match="shapes do not agree"):
+        wire.pack_host(cdf, maxima, lengths, payload, 1, 3, 300)
+
+
+# --------------------------------------------------------------------------- #
+# GPU
+# --------------------------------------------------------------------------- #
+DEV = "cuda:0"
+
+
+def _bits(t):
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_device_blobs_equal_the_host_definition(dtype):
+    from cachegen_amd import codec
+    from cachegen_amd.kvgen import make_kv
+    L, T, H, D, S = 2, 900, 4, 64, 512
+    kv = make_kv(L, T, H, D, seed=11, device=DEV, dtype=dtype)
+    bins = torch.tensor([32.0, 16.0])
+    enc = codec.encode_kv(kv, bins, bins, chunk_tokens=S)
+    blobs = wire.pack_chunks(enc)
+    assert len(blobs) == 2
+    bounds = enc.sub_boundaries()
+    for i, blob in enumerate(blobs):
+        t0, t1 = i * S, min((i + 1) * S, T)
+        g0, g1 = 2 * i, min(2 * i + 2, enc.lengths.shape[0])
+        want = wire.pack_host(enc.cdf[i:i + 1].cpu().numpy(), _bits(enc.maxima[:, :, t0:t1]),
+                              enc.lengths[g0:g1].cpu().numpy(), enc.payload[bounds[g0]:bounds[g1]].cpu().numpy(),
+                              H, D, S, bf16_maxima=dtype == torch.bfloat16)
+        assert blob == want
+    whole = wire.pack_chunks(enc, per_chunk=False)
+    assert len(whole) == 1
+    want = wire.pack_host(enc.cdf.cpu().numpy(), _bits(enc.maxima), enc.lengths.cpu().numpy(),
+                          enc.payload[:enc.total_bytes()].cpu().numpy(), H, D, S,
+                          bf16_maxima=dtype == torch.bfloat16)
+    assert whole[0] == want
+    # back on the device: the sections are the encoder's tensors
+    h, cdf, maxima, lengths, payload = wire.unpack_to_device(whole[0], DEV)
+    assert torch.equal(cdf, enc.cdf) and torch.equal(lengths, enc.lengths)
+    assert maxima.dtype == dtype and torch.equal(maxima.view(torch.int16), enc.maxima.view(torch.int16))
+    assert torch.equal(payload, enc.payload[:enc.total_bytes()])
+    out = codec.decode_kv(cdf, maxima, codec.scan_lengths(lengths), payload, bins, bins, L, T, H, D, S,
+                          out_dtype=dtype)
+    assert torch.equal(out.view(torch.int16), codec.decode_encoded(enc, bins, bins, out_dtype=dtype).view(torch.int16))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fmt", ["vllm", "huggingface"])
+def test_flat_serde_decodes_to_the_same_tensor_as_the_pickle_serde(fmt):
+    from cachegen_amd.config import LMCacheEngineConfig, LMCacheEngineMetadata
+    from cachegen_amd.kvgen import make_kv
+    from cachegen_amd.serde import CreateSerde
+    config = LMCacheEngineConfig.from_defaults(chunk_size=256)
+    meta = LMCacheEngineMetadata("lmsys/longchat-7b-16k", 1, 0, fmt)
+    s_ref, d = CreateSerde("cachegen", config, meta)
+    s_flat, _ = CreateSerde("cachegen-flat", config, meta)
+    for ntok in (256, 77, 600):
+        kv = make_kv(32, ntok, 2, 64, seed=ntok, device=DEV)
+        if fmt == "huggingface":
+            kv = kv.permute(0, 1, 3, 2, 4).contiguous()
+        a, b = s_ref.to_bytes(kv), s_flat.to_bytes(kv)
+        assert wire.is_flat(b) and not wire.is_flat(a)
+        assert len(b) < len(a) + 512
+        ta, tb = d.from_bytes(a), d.from_bytes(b)
+        assert ta.shape == kv.shape and ta.dtype == tb.dtype
+        assert torch.equal(ta.view(torch.int16), tb.view(torch.int16))
+    bad = bytearray(b)
+    h = wire.read_header(b)
+    off = h["geometry"]["lengths"][0]
+    bad[off:off + 4] = struct.pack("<i", 1 + struct.unpack_from("<i", b, off)[0])
+    with pytest.raises(ValueError, match="sum of the stream lengths"):
+        d.from_bytes(bytes(bad))

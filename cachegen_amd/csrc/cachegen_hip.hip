@@ -664,7 +664,11 @@ __device__ __forceinline__ StreamId locate(const StreamGrid &sg)
 }
 
 // ---- encoder (enc_new.cu:21-97, 253-307) -------------------------------------------
-// Bits are collected MSB-first in a 32-bit accumulator and leave as big-endian words.
+// Bits are collected MSB-first in a 64-bit accumulator and leave as big-endian 32-bit words.
+// Every lane of a wavefront runs the store code whenever one lane has a word ready, so words
+// are written at fixed points, once per two symbols, instead of whenever a lane's
+// accumulator fills; the accumulator takes the two symbols in between (a put that would not
+// fit writes a word first).
 // The E1/E2 run of a symbol is emitted at once: the n1 = clz(low ^ high) leading bits
 // agree, and the pending complements go in after the first of them, which in arithmetic
 // is  bits + ((2^pend - 1) << (n1 - 1))  over n1 + pend bits.  The E3 run k is the number
@@ -674,9 +678,10 @@ __device__ __forceinline__ StreamId locate(const StreamGrid &sg)
 template <bool ALIGNED>
 struct BitWriter {
     uint8_t *wptr;          // where the next word goes
+    int wstride;            // bytes from one word of the stream to the next (4: contiguous)
     int cap;
     int nbytes;
-    uint32_t acc;
+    uint64_t acc;           // the low `nacc` bits are waiting to be written; bits above are stale
     int nacc;
 
     // the last words of a stream that does not fit its slot: keep what fits
@@ -700,23 +705,25 @@ struct BitWriter {
         } else {
             store_clipped(word);
         }
-        wptr += 4;
+        wptr += wstride;
         nbytes += 4;
+    }
+
+    // write one word if 32 bits are waiting
+    __device__ __forceinline__ void flush_word()
+    {
+        if (nacc >= 32) {
+            store_word((uint32_t)(acc >> (nacc - 32)));
+            nacc -= 32;
+        }
     }
 
     // append the low m bits of v (v < 2^m), 0 <= m <= 32 (m = 0 needs v = 0)
     __device__ __forceinline__ void put(uint32_t v, int m)
     {
-        const int tot = nacc + m;
-        if (tot >= 32) {
-            const uint32_t vl = v << ((32 - m) & 31);
-            store_word(__builtin_amdgcn_alignbit(acc, vl, (uint32_t)nacc));
-            nacc = tot - 32;
-            acc = v & ((1u << nacc) - 1u);
-        } else {
-            acc = (acc << m) | v;
-            nacc = tot;
-        }
+        if (__builtin_expect(nacc + m > 64, 0)) flush_word();       // more than 32 are waiting then
+        acc = (acc << m) | v;
+        nacc += m;
     }
 
     // one bit, then `count` copies of its complement (any count): the general form of
@@ -727,6 +734,7 @@ struct BitWriter {
         int pm = 1;
         for (;;) {
             put(pv, pm);
+            flush_word();
             if (count == 0) break;
             pm = count < 32u ? (int)count : 32;
             pv = bit ? 0u : (pm == 32 ? 0xFFFFFFFFu : ((1u << pm) - 1u));
@@ -734,11 +742,14 @@ struct BitWriter {
         }
     }
 
-    // write the partial accumulator (enc_new.cu:42-55); returns the stream length
+    // write what is left, the last partial word byte by byte (enc_new.cu:42-55); returns
+    // the stream length
     __device__ __forceinline__ int finish()
     {
+        flush_word();
+        flush_word();
         if (nacc > 0) {
-            uint32_t r = acc << (32 - nacc);
+            uint32_t r = (uint32_t)(acc << (32 - nacc));
             for (int left = nacc, j = 0; left > 0; left -= 8, ++j) {
                 if (nbytes < cap) wptr[j] = (uint8_t)(r >> 24);
                 nbytes++;
@@ -760,7 +771,7 @@ struct RangeEncoder {
     uint32_t low, span, pend;
     BitWriter<ALIGNED> w;
 
-    __device__ __forceinline__ void init(const uint16_t *column, int lp, uint8_t *dst, int cap)
+    __device__ __forceinline__ void init(const uint16_t *column, int lp, uint8_t *dst, int wstride, int cap)
     {
         col = column;
         smax = (uint32_t)(lp - 2);
@@ -768,18 +779,22 @@ struct RangeEncoder {
         span = 0;
         pend = 0;
         w.wptr = dst;
+        w.wstride = wstride;
         w.cap = cap;
         w.nbytes = 0;
         w.acc = 0;
         w.nacc = 0;
     }
 
+    // SENTINEL: symbol smax may occur, whose upper bound is 2^16 and not the table's last
+    // entry (enc_new.cu:270)
+    template <bool SENTINEL>
     __device__ __forceinline__ void put_symbol(uint32_t s)
     {
         s = s < smax ? s : smax;                        // keep table reads inside the table
         const uint32_t c_lo = col[s * BS];
         const uint32_t c_next = col[s * BS + BS];
-        const uint32_t c_hi = s == smax ? 0x10000u : c_next;    // the table ends at 2^16 (enc_new.cu:270)
+        const uint32_t c_hi = (SENTINEL && s == smax) ? 0x10000u : c_next;
         uint32_t t_lo, width;
         if (__builtin_expect(span == 0, 0)) {
             t_lo = c_lo << 16;
@@ -793,20 +808,23 @@ struct RangeEncoder {
         const uint32_t high = low + width - 1u;
 
         const int n1 = __builtin_clz(low ^ high);       // low < high always
-        if (n1 > 0) {
-            const uint32_t bits = low >> ((32 - n1) & 31);           // the n1 agreed bits
-            if (__builtin_expect(pend + (uint32_t)n1 > 32u, 0)) {
-                w.bit_and_run(bits >> (n1 - 1), pend);
-                w.put(bits & ((1u << (n1 - 1)) - 1u), n1 - 1);
-            } else {
-                const uint32_t fill = ((1u << (pend & 31)) - 1u) << (n1 - 1);
-                w.put(bits + fill, n1 + (int)pend);
-            }
-            pend = 0;
+        // the n1 agreed bits (none if n1 = 0) with the pending complements after the first
+        const uint32_t pe = n1 > 0 ? pend : 0u;
+        const int m = n1 + (int)pe;
+        if (__builtin_expect(m > 32, 0)) {
+            const uint32_t bits = low >> ((32 - n1) & 31);
+            w.bit_and_run(bits >> (n1 - 1), pe);
+            w.put(bits & ((1u << (n1 - 1)) - 1u), n1 - 1);
+        } else {
+            const uint32_t bits = __builtin_amdgcn_ubfe(low, (uint32_t)(32 - n1), (uint32_t)n1);
+            const uint32_t fill = ((1u << (pe & 31)) - 1u) << ((n1 - 1) & 31);
+            w.put(bits + fill, m);
         }
-        const int k = __builtin_clz(~((low & ~high) << ((n1 + 1) & 31)));
-        const int n = (n1 + k) & 31;
-        pend += (uint32_t)k;
+        // E3 run: leading zeros of (~low | high) below the first differing bit
+        const uint32_t z = ((low & high) | ~low) << ((n1 + 1) & 31);
+        const int k = __builtin_clz(z);
+        const int n = n1 + k;
+        pend = pend - pe + (uint32_t)k;
         low = (low << n) & 0x7FFFFFFFu;
         span = width << n;
     }
@@ -826,12 +844,21 @@ struct EncodeArgs {
     int64_t s0, s1, s2;
     const uint32_t *sym4;   // or packed symbols
     int64_t nsub;
-    uint8_t *out;           // out[row*o0 + channel*o1 + byte], or one `cap`-byte slot per
-    int64_t o0, o1;         // stream in stream order (SLOTS)
+    uint8_t *out;           // out[row*o0 + channel*o1 + byte], or the scratch tiles (SLOTS)
+    int64_t o0, o1;
     int32_t cap;
     int32_t *lengths;       // [sub][row][channel]
     int32_t *status;        // may be null
+    const float *key_bins, *value_bins;     // float32 [L] each, or null when the levels are not known
+    int64_t L;
     StreamGrid sg;
+};
+
+constexpr int kSlotTile = 256;      // streams per tile of the encoder's scratch
+
+template <bool B>
+struct BoolTag {
+    static constexpr bool value = B;
 };
 
 // PACKED: symbols come from sym4.  FUSE_CDF (PACKED only, one sub-chunk per chunk): the
@@ -892,36 +919,62 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
 
     RangeEncoder<BS, ALIGNED> enc;
     const int64_t stream = (id.sub * a.sg.rows + id.row) * a.sg.nc + id.ch;
-    enc.init(col, lp, SLOTS ? a.out + stream * a.cap : a.out + id.row * a.o0 + id.ch * a.o1, a.cap);
+    // SLOTS: the scratch is cut into tiles of kSlotTile streams; word w of a tile's stream t is
+    // the tile's word w * kSlotTile + t, so that the words the lanes of a wavefront write, and
+    // the words the compaction reads, lie side by side
+    if (SLOTS)
+        enc.init(col, lp, a.out + (stream / kSlotTile) * ((int64_t)kSlotTile * a.cap) + (stream % kSlotTile) * 4,
+                 kSlotTile * 4, a.cap);
+    else
+        enc.init(col, lp, a.out + id.row * a.o0 + id.ch * a.o1, 4, a.cap);
 
-    if (PACKED) {
-        for (int h = 0; h * 32 < nwords; ++h) {
-            load_half(h);
-            const int wn = nwords - h * 32 < 32 ? nwords - h * 32 : 32;
+    // The row's alphabet (2C + 1 symbols for `bins` levels, encoder.py:44-52) may leave the
+    // table's last symbol unused; then its special upper bound is never needed.  Uniform
+    // over the block.
+    bool sentinel = true;
+    if (PACKED && a.key_bins) {
+        const int64_t kvi = id.row / a.L, l = id.row - kvi * a.L;
+        const float cq = floorf((kvi ? a.value_bins : a.key_bins)[l] * 0.5f) - 1.0f;
+        sentinel = !(cq >= 0.0f && 2.0f * cq + 1.0f <= (float)(lp - 2));
+    }
+
+    auto code = [&](auto tag) {
+        constexpr bool SENTINEL = decltype(tag)::value;
+        if (PACKED) {
+            for (int h = 0; h * 32 < nwords; ++h) {
+                load_half(h);
+                const int wn = nwords - h * 32 < 32 ? nwords - h * 32 : 32;
 #pragma unroll 1
-            for (int w = 0; w < wn; ++w) {
-                const uint32_t v = words[w];
+                for (int w = 0; w < wn; ++w) {
+                    const uint32_t v = words[w];
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    if ((h * 32 + w) * 4 + j < id.n) enc.put_symbol((v >> (8 * j)) & 0xFFu);
+                    for (int j = 0; j < 4; ++j) {
+                        if ((h * 32 + w) * 4 + j < id.n) enc.template put_symbol<SENTINEL>((v >> (8 * j)) & 0xFFu);
+                        if (j & 1) enc.w.flush_word();
+                    }
+                }
+            }
+        } else {
+            const uint8_t *sp = a.sym + id.row * a.s0 + id.t0 * a.s1 + id.ch * a.s2;
+            uint32_t nxt[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) nxt[j] = (j < id.n) ? sp[(int64_t)j * a.s1] : 0u;
+            for (int i0 = 0; i0 < id.n; i0 += 8) {
+                uint32_t cur[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) cur[j] = nxt[j];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) nxt[j] = (i0 + 8 + j < id.n) ? sp[(int64_t)(i0 + 8 + j) * a.s1] : 0u;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    if (i0 + j < id.n) enc.template put_symbol<SENTINEL>(cur[j]);
+                    if (j & 1) enc.w.flush_word();
+                }
             }
         }
-    } else {
-        const uint8_t *sp = a.sym + id.row * a.s0 + id.t0 * a.s1 + id.ch * a.s2;
-        uint32_t nxt[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) nxt[j] = (j < id.n) ? sp[(int64_t)j * a.s1] : 0u;
-        for (int i0 = 0; i0 < id.n; i0 += 8) {
-            uint32_t cur[8];
-#pragma unroll
-            for (int j = 0; j < 8; ++j) cur[j] = nxt[j];
-#pragma unroll
-            for (int j = 0; j < 8; ++j) nxt[j] = (i0 + 8 + j < id.n) ? sp[(int64_t)(i0 + 8 + j) * a.s1] : 0u;
-#pragma unroll
-            for (int j = 0; j < 8; ++j)
-                if (i0 + j < id.n) enc.put_symbol(cur[j]);
-        }
-    }
+    };
+    if (PACKED && !sentinel) code(BoolTag<false>());
+    else code(BoolTag<true>());
     const int len = enc.finish();
     a.lengths[stream] = len;
     if (len > a.cap && a.status) atomicOr(a.status, 1);
@@ -1137,6 +1190,10 @@ __device__ __forceinline__ void decode_symbol(const DecodeArgs &a, DecodeLane &s
     } else {
         const float q = *(lds_f32 *)(p + s.lutoff);
         float v = __fmul_rn(q, rm);
+        // the product is rounded to float32 before it is rounded to 16 bits (decoder.py:28-34
+        // works in float32): keep the compiler from merging the two into one mixed-precision
+        // multiply, which rounds once and turns -0 into +0
+        asm volatile("" : "+v"(v));
         if (SAFE && a.delta_group > 0) {             // uniform over the block
             if (s.phase == 0) s.anchor = v;
             else v = __fadd_rn(v, s.anchor);
@@ -1345,21 +1402,23 @@ __global__ __launch_bounds__(kScanThreads) void scan_apply_kernel(
 }
 
 // ------------------------------------------------------------------------------------
-// collect_bytes (encoder.py:209-222), output-centric: a block owns 256 consecutive
-// streams, i.e. one contiguous range of the payload.  Every thread assembles aligned
-// 32-bit words of that range: it finds the stream of the word's first byte by binary
-// search over the block's offsets (in LDS); a word that lies inside one stream is two
-// aligned loads from that stream's slot and a funnel shift, a word that straddles streams
-// or the ends of the range is gathered and stored byte by byte, so neighbouring blocks
-// never write the same byte.  All positions are 32-bit offsets from the range's start.
+// collect_bytes (encoder.py:209-222).  A block owns 256 consecutive streams, i.e. one
+// contiguous range of the payload, and assembles it in LDS, 16 KiB at a time: every thread
+// copies its own stream from its slot to the stream's place in the range (aligned words
+// through a funnel shift, single bytes at the two ends), then the block writes the tile out
+// as aligned 32-bit words.  Only the first and last word of a block's range are written
+// byte by byte, so neighbouring blocks never write the same byte.  All positions are
+// 32-bit offsets from the range's start.
 // ------------------------------------------------------------------------------------
 constexpr int kCompactStreams = 256;
+constexpr int kCompactTile = 16384;
 
 __global__ __launch_bounds__(256) void compact_streams_kernel(
     const uint8_t *__restrict__ slots, int32_t cap, const int64_t *__restrict__ offsets,
     int64_t nstreams, uint8_t *__restrict__ payload, int64_t payload_cap, int32_t skew, int32_t *status)
 {
     __shared__ int32_t rel[kCompactStreams + 1];       // stream offsets relative to the block's first byte
+    __shared__ uint32_t buf[kCompactTile / 4];
     const int tid = threadIdx.x;
     const int64_t sbase = (int64_t)blockIdx.x * kCompactStreams;
     const int count = (nstreams - sbase < kCompactStreams) ? (int)(nstreams - sbase) : kCompactStreams;
@@ -1372,38 +1431,56 @@ __global__ __launch_bounds__(256) void compact_streams_kernel(
         if (tid == 0 && status) atomicOr(status, 2);
         return;
     }
-    const uint8_t *src = slots + sbase * (int64_t)cap;
-    uint8_t *dst = payload + o0;
-    // words are aligned in memory: `lead` bytes of the first word lie before the range
+    // x = position in the range + lead: aligned words of the payload are at multiples of 4
     const int lead = (int)((o0 + skew) & 3);
-    const int nwords = (lead + total + 3) >> 2;
-    int nsteps = 0;
-    while ((1 << nsteps) < count) ++nsteps;
-    for (int w = tid; w < nwords; w += 256) {
-        const int p0 = 4 * w - lead;                   // may be negative for w = 0
-        const int pfirst = p0 < 0 ? 0 : p0;
-        const int pend = p0 + 4 < total ? p0 + 4 : total;
-        int lo = 0, hi = count - 1;                    // largest s with rel[s] <= pfirst
-        for (int step = 0; step < nsteps; ++step) {
-            const int mid = (lo + hi + 1) >> 1;
-            const bool le = rel[mid] <= pfirst;
-            lo = le ? mid : lo;
-            hi = le ? hi : mid - 1;
-        }
-        int s = lo;
-        if (pend - pfirst == 4 && pfirst + 3 < rel[s + 1]) {
-            const int q = pfirst - rel[s];
-            const uint8_t *slot = src + s * cap;       // 32-bit offset: 256 streams * cap bytes
-            const int at = q & ~3, sh = (q & 3) * 8;
-            const uint32_t w_lo = *reinterpret_cast<const uint32_t *>(slot + at);
-            const uint32_t w_hi = (sh != 0) ? *reinterpret_cast<const uint32_t *>(slot + at + 4) : 0u;
-            *reinterpret_cast<uint32_t *>(dst + p0) = __builtin_amdgcn_alignbit(w_hi, w_lo, (uint32_t)sh);
-        } else {
-            for (int p = pfirst; p < pend; ++p) {
-                while (p >= rel[s + 1]) ++s;           // streams are at least one byte long
-                dst[p] = src[s * cap + (p - rel[s])];
+    uint8_t *const dst = payload + o0 - lead;
+    const int end = lead + total;
+    const int my0 = rel[tid] + lead, my1 = rel[tid + 1] + lead;     // rel[] is padded with the total
+    // word k of this thread's stream (see encode_streams_kernel: tiles of kSlotTile streams)
+    const uint32_t *const words = reinterpret_cast<const uint32_t *>(slots + sbase * (int64_t)cap) + tid;
+    const int kmax = (my1 - my0 - 1) >> 2;             // last word that holds bytes of the stream
+    uint8_t *const bytes = reinterpret_cast<uint8_t *>(buf);
+
+    for (int t0 = 0; t0 < end; t0 += kCompactTile) {
+        const int t1 = t0 + kCompactTile < end ? t0 + kCompactTile : end;
+        const int xs = my0 > t0 ? my0 : t0;
+        const int xe = my1 < t1 ? my1 : t1;
+        // aligned words j of the range that hold bytes [xs, xe) of this stream, eight at a time:
+        // word j is stream bytes 4j - my0 .. +3, i.e. two stream words through a funnel shift
+        for (int j = xs >> 2; 4 * j < xe; j += 8) {
+            const int q = 4 * j - my0;                 // may be negative for the stream's first word
+            const int k = q >> 2;
+            const uint32_t sh = (uint32_t)(q & 3) * 8u;
+            const int left = ((xe + 3) >> 2) - j;      // words still to produce
+            uint32_t wv[9];
+#pragma unroll
+            for (int u = 0; u < 9; ++u)
+                wv[u] = (k + u >= 0 && k + u <= kmax && u <= left) ? words[(k + u) * kSlotTile] : 0u;
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                if (u >= left) break;
+                const uint32_t v = __builtin_amdgcn_alignbit(wv[u + 1], wv[u], sh);
+                const int x0 = 4 * (j + u);
+                if (x0 >= xs && x0 + 4 <= xe) {
+                    buf[(x0 - t0) >> 2] = v;
+                } else {
+                    for (int c = 0; c < 4; ++c)
+                        if (x0 + c >= xs && x0 + c < xe) bytes[x0 + c - t0] = (uint8_t)(v >> (8 * c));
+                }
             }
         }
+        __syncthreads();
+        for (int w = (t0 >> 2) + tid; 4 * w < t1; w += 256) {
+            const int x0 = 4 * w;
+            const uint32_t v = buf[w - (t0 >> 2)];
+            if (x0 >= lead && x0 + 4 <= end) {
+                *reinterpret_cast<uint32_t *>(dst + x0) = v;
+            } else {
+                for (int j = 0; j < 4; ++j)
+                    if (x0 + j >= lead && x0 + j < end) dst[x0 + j] = (uint8_t)(v >> (8 * j));
+            }
+        }
+        __syncthreads();
     }
 }
 
@@ -1768,7 +1845,7 @@ size_t cg_encode_kv_workspace(int64_t L, int64_t T, int64_t C, int64_t chunk_tok
     const int64_t nsub = cg_num_subchunks(T, chunk_tokens);
     const int64_t nstreams = nsub * 2 * L * C;
     size_t total = align_up((size_t)nstreams * kSub, 256);        // symbols: a 256-token slot per stream
-    total += align_up((size_t)nstreams * kStreamCap, 256);        // encoder scratch: a slot per stream
+    total += (size_t)ceil_div(nstreams, kSlotTile) * kSlotTile * kStreamCap;   // encoder scratch: whole tiles of slots
     total += cg_scan_workspace(nstreams);
     return total;
 }
@@ -1798,8 +1875,8 @@ int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int
     uint8_t *ws = static_cast<uint8_t *>(workspace);
     uint8_t *symbols = ws;
     ws += align_up((size_t)nstreams * kSub, 256);
-    uint8_t *scratch = ws;     // one kStreamCap-byte slot per stream
-    ws += align_up((size_t)nstreams * kStreamCap, 256);
+    uint8_t *scratch = ws;     // kStreamCap bytes per stream, in tiles of kSlotTile word-interleaved streams
+    ws += (size_t)ceil_div(nstreams, kSlotTile) * kSlotTile * kStreamCap;
     void *scan_scratch = ws;
     uint16_t *tables = reinterpret_cast<uint16_t *>(cdf);
 
@@ -1815,6 +1892,9 @@ int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int
     a.cap = kStreamCap;
     a.lengths = lengths;
     a.status = status;
+    a.key_bins = key_bins;
+    a.value_bins = value_bins;
+    a.L = L;
     int64_t nblocks;
     if (int rc = make_grid(rows, C, T, chunk_tokens, nsub, block, a.sg, nblocks)) return rc;
     const size_t shmem = (size_t)lp * block * sizeof(uint16_t);

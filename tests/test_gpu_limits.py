@@ -109,3 +109,61 @@ def test_payload_buffer_too_small_is_reported():
     with pytest.raises(RuntimeError, match="payload buffer too small"):
         small.check()
     assert (base[total - 1:] == 0xEE).all()                 # nothing written past the buffer
+
+
+@pytest.mark.parametrize("dtype,dt", [(torch.float16, 0), (torch.bfloat16, 1)])
+def test_high_entropy_streams_match_oracle(oracle, dtype, dt):
+    """White-noise KV: about 4 bits per symbol, so a block of 256 streams holds well over
+    16 KiB of payload and the compaction works through several tiles; 300 tokens make the
+    second sub-chunk short, 5 layers an odd number of rows."""
+    codec, _ = _mods()
+    torch.manual_seed(3)
+    L, T, H, D = 5, 300, 4, 128
+    kv = torch.randn((L, 2, T, H, D), dtype=torch.float32).to(dtype)
+    kb = torch.tensor([32.0, 32.0, 16.0, 32.0, 16.0])
+    vb = torch.tensor([32.0, 16.0, 16.0, 32.0, 32.0])
+    enc = codec.encode_kv(kv.to(DEV), kb, vb, chunk_tokens=T)
+    enc.check()
+    flat = kv.reshape(L, 2, T, H * D).contiguous().view(torch.int16).numpy().view(np.uint16)
+    want = oracle.encode_function(flat, kb.numpy(), vb.numpy(), dt)
+    assert np.array_equal(enc.cdf[0].cpu().numpy().view(np.uint16), want["cdf"])
+    bounds = enc.sub_boundaries()
+    assert (bounds[1] - bounds[0]) / (2 * L * H * D / 256) > 20000      # bytes per block of 256 streams
+    for g, (data, lengths, ntok) in enumerate(want["data_chunks"]):
+        assert np.array_equal(enc.lengths[g].cpu().numpy(), lengths)
+        assert np.array_equal(enc.payload[bounds[g]:bounds[g + 1]].cpu().numpy(), data)
+    out = codec.decode_encoded(enc, kb, vb, out_dtype=dtype)
+    _, ref = oracle.decode_function(want, kb.numpy(), vb.numpy(), dt, dt)
+    got = out.cpu().reshape(L, 2, T, H * D).contiguous().view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(got, ref)
+
+
+def test_nan_and_infinite_rows_match_oracle(oracle):
+    """Rows whose maximum is infinite or NaN take the decoder's careful path; every other
+    row of the same tensor takes the fast one."""
+    codec, _ = _mods()
+    torch.manual_seed(4)
+    L, T, H, D = 2, 64, 2, 64
+    kv = torch.randn((L, 2, T, H, D), dtype=torch.float32)
+    kv[0, 0, 3, 0, 5] = float("inf")
+    kv[1, 1, 9, 1, 7] = float("nan")
+    kv[0, 1, 11, 0, 0] = float("-inf")
+    kv[1, 0, 20] = 0.0                                   # an all-zero row: 0 * inf
+    bins = torch.tensor([32.0, 16.0])
+    for dtype, dt in ((torch.float16, 0), (torch.bfloat16, 1)):
+        x = kv.to(dtype)
+        enc = codec.encode_kv(x.to(DEV), bins, bins, chunk_tokens=T)
+        enc.check()
+        flat = x.reshape(L, 2, T, H * D).contiguous().view(torch.int16).numpy().view(np.uint16)
+        want = oracle.encode_function(flat, bins.numpy(), bins.numpy(), dt)
+        assert np.array_equal(enc.payload[:enc.total_bytes()].cpu().numpy(), want["data_chunks"][0][0])
+        for out_dtype, odt in ((torch.float16, 0), (torch.bfloat16, 1)):
+            out = codec.decode_encoded(enc, bins, bins, out_dtype=out_dtype)
+            _, ref = oracle.decode_function(want, bins.numpy(), bins.numpy(), dt, odt)
+            got = out.cpu().reshape(L, 2, T, H * D).contiguous().view(torch.int16).numpy().view(np.uint16)
+            # 0 * inf has no defined sign or payload (x86 gives the negative default NaN, the GPU
+            # the positive one): NaNs must be in the same places, every other value bit-equal
+            inf_bits = 0x7C00 if odt == 0 else 0x7F80
+            nan_got, nan_ref = (got & 0x7FFF) > inf_bits, (ref & 0x7FFF) > inf_bits
+            assert np.array_equal(nan_got, nan_ref), (dtype, out_dtype)
+            assert nan_ref.any() and np.array_equal(got[~nan_ref], ref[~nan_ref]), (dtype, out_dtype)

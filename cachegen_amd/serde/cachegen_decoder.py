@@ -63,8 +63,26 @@ class CacheGenDeserializer(Deserializer):
         float16 [num_layers, 2, num_heads, num_tokens, head_size] for "huggingface"
         (cachegen_decoder.py:144-173).  Decode, dequantization, cast and layout are one
         kernel.  Blobs in the flat container of `wire` are recognised by their magic."""
+        return self._decode(bs, None)
+
+    def from_bytes_into(self, bs: bytes, out: torch.Tensor) -> torch.Tensor:
+        """Decodes `bs` straight into `out`: a tensor, or a view into a larger one, of the
+        chunk's shape in this deserializer's layout, float16 or bfloat16 (not in the reference,
+        whose callers concatenate the decoded chunks)."""
+        return self._decode(bs, out)
+
+    def chunk_shape(self, bs: bytes):
+        """Shape `from_bytes(bs)` would have, read from a flat container's header without
+        decoding; None for a pickle container."""
+        if not wire.is_flat(bs):
+            return None
+        h = wire.read_header(bs)
+        L, T, H, D = h["num_layers"], h["num_tokens"], h["num_heads"], h["head_size"]
+        return (L, 2, T, H, D) if self.fmt == "vllm" else (L, 2, H, T, D)
+
+    def _decode(self, bs, out):
         if wire.is_flat(bs):
-            return self._from_flat(bs)
+            return self._from_flat(bs, out)
         encoder_output = CacheGenGPUEncoderOutput.from_bytes(bs)
         cdf = encoder_output.cdf.cuda()
         max_k = encoder_output.max_tensors_key.cuda()
@@ -81,9 +99,9 @@ class CacheGenDeserializer(Deserializer):
         maxima = torch.stack([max_k.reshape(nlayers, ntokens), max_v.reshape(nlayers, ntokens)])
         return codec.decode_kv(cdf.unsqueeze(0), maxima, offsets, payload, self.key_bins,
                                self.value_bins, nlayers, ntokens, encoder_output.num_heads,
-                               encoder_output.head_size, chunk_tokens=ntokens, fmt=self.fmt)
+                               encoder_output.head_size, chunk_tokens=ntokens, fmt=self.fmt, out=out)
 
-    def _from_flat(self, bs) -> torch.Tensor:
+    def _from_flat(self, bs, out=None) -> torch.Tensor:
         h, cdf, maxima, lengths, payload = wire.unpack_to_device(bs, self.key_bins.device)
         if h["num_layers"] != self.key_bins.numel():
             raise ValueError("blob has %d layers, this deserializer's model %d"
@@ -94,4 +112,5 @@ class CacheGenDeserializer(Deserializer):
             raise ValueError("wire container: payload size is not the sum of the stream lengths")
         return codec.decode_kv(cdf, maxima, offsets, payload, self.key_bins, self.value_bins,
                                h["num_layers"], h["num_tokens"], h["num_heads"], h["head_size"],
-                               chunk_tokens=h["chunk_tokens"], fmt=self.fmt, delta_group=h["delta_group"])
+                               chunk_tokens=h["chunk_tokens"], fmt=self.fmt, delta_group=h["delta_group"],
+                               out=out)

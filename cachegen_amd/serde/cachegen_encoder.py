@@ -83,3 +83,23 @@ class CacheGenSerializer(Serializer):
         output = encode_function(tensor.cuda(), self.cachegen_config, self.key_bins,
                                  self.value_bins, ntokens)
         return output.to_bytes()
+
+    def to_bytes_chunks(self, tensor: torch.Tensor, chunk_size: int):
+        """One blob per `chunk_size` tokens of `tensor` (same layouts as `to_bytes`), each equal
+        to what `to_bytes` returns for that slice; all chunks are encoded in one pass over the
+        tensor (not in the reference, whose callers loop over `to_bytes`)."""
+        if self.fmt == "huggingface":
+            tensor = tensor.permute(0, 1, 3, 2, 4)
+        num_heads, head_size = tensor.shape[-2:]
+        enc = codec.encode_kv(tensor.cuda(), self.key_bins, self.value_bins, chunk_tokens=chunk_size)
+        if self.wire_format == "flat":
+            return wire.pack_chunks(enc)
+        enc.check()
+        bounds = enc.sub_boundaries()
+        blobs = []
+        for i in range(enc.num_chunks):
+            cdf, max_k, max_v, subs = enc.chunk(i, bounds)
+            data_chunks = [CacheGenGPUBytestream(bytestream=b, bytestream_lengths=l, ntokens=n) for b, l, n in subs]
+            blobs.append(CacheGenGPUEncoderOutput(data_chunks, cdf, max_tensors_key=max_k, max_tensors_value=max_v,
+                                                  num_heads=num_heads, head_size=head_size).to_bytes())
+        return blobs

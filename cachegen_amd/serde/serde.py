@@ -33,6 +33,9 @@ class SerializerDebugWrapper(Serializer):
         logger.debug("Serialization took %.2f seconds", time.perf_counter() - start)
         return bs
 
+    def __getattr__(self, name):           # whatever else the wrapped serializer offers
+        return getattr(self.s, name)
+
 
 class DeserializerDebugWrapper(Deserializer):
     def __init__(self, d: Deserializer):
@@ -43,3 +46,6 @@ class DeserializerDebugWrapper(Deserializer):
         ret = self.d.from_bytes(bs)
         logger.debug("Deserialization took %.2f ms", (time.perf_counter() - start) * 1000)
         return ret
+
+    def __getattr__(self, name):
+        return getattr(self.d, name)

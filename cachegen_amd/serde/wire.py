@@ -176,8 +176,9 @@ def pack_chunks(enc, first_chunk: int = 0, num_chunks: Optional[int] = None, per
         t0, t1 = c0 * S, min(c1 * S, T)
         g0, g1 = c0 * spc, min(c1 * spc, enc.lengths.shape[0])
         nbytes = bounds[g1] - bounds[g0]
-        geo = geometry(L, t1 - t0, H, D, S, enc.max_bins, nbytes)
-        head = write_header(L, t1 - t0, H, D, S, enc.max_bins, enc.delta_group, g1 - g0, nbytes, bf16)
+        table_tokens = min(S, t1 - t0)          # a short last chunk is a blob of its own length
+        geo = geometry(L, t1 - t0, H, D, table_tokens, enc.max_bins, nbytes)
+        head = write_header(L, t1 - t0, H, D, table_tokens, enc.max_bins, enc.delta_group, g1 - g0, nbytes, bf16)
         plans.append((total, geo, head, (c0, c1, t0, t1, g0, g1)))
         total += geo["total"][0]
     dev = enc.payload.device

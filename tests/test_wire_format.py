@@ -113,7 +113,7 @@ def test_device_blobs_equal_the_host_definition(dtype):
         g0, g1 = 2 * i, min(2 * i + 2, enc.lengths.shape[0])
         want = wire.pack_host(enc.cdf[i:i + 1].cpu().numpy(), _bits(enc.maxima[:, :, t0:t1]),
                               enc.lengths[g0:g1].cpu().numpy(), enc.payload[bounds[g0]:bounds[g1]].cpu().numpy(),
-                              H, D, S, bf16_maxima=dtype == torch.bfloat16)
+                              H, D, min(S, t1 - t0), bf16_maxima=dtype == torch.bfloat16)
         assert blob == want
     whole = wire.pack_chunks(enc, per_chunk=False)
     assert len(whole) == 1

@@ -136,10 +136,21 @@ def cpu_baseline(kv_cpu, kbins, vbins, chunk, sample_tokens):
         oracle.decode_function(e, kb, vb)
     t2 = time.perf_counter()
     nbytes = 2 * L * n * H * D * 2
+    # the same code on one core, on the first chunk only
+    one = flat[:, :, :min(chunk, n)]
+    oracle.set_threads(1)
+    s0 = time.perf_counter()
+    e1 = oracle.encode_function(one, kb, vb)
+    oracle.decode_function(e1, kb, vb)
+    s1 = time.perf_counter()
+    oracle.set_threads(cores)
+    one_bytes = 2 * L * one.shape[2] * H * D * 2
     return dict(value=round(2 * nbytes / (t2 - t0) / 1e9, 4), unit="GB/s", cores=cores, kind="port",
                 sample="first %d tokens of the workload (%d chunks of %d): %.1f MB fp16, C oracle with OpenMP"
                        % (n, len(encs), chunk, nbytes / 1e6),
-                encode_GBps=round(nbytes / (t1 - t0) / 1e9, 4), decode_GBps=round(nbytes / (t2 - t1) / 1e9, 4))
+                encode_GBps=round(nbytes / (t1 - t0) / 1e9, 4), decode_GBps=round(nbytes / (t2 - t1) / 1e9, 4),
+                one_core_GBps=round(2 * one_bytes / (s1 - s0) / 1e9, 4),
+                one_core_sample="first chunk (%d tokens, %.1f MB fp16)" % (one.shape[2], one_bytes / 1e6))
 
 
 def main():
@@ -257,6 +268,8 @@ def main():
         "decode_GBps": round(kv_bytes / (dec_avg * 1e-3) / 1e9, 3),
         "encode_ms": round(enc_avg, 4),
         "decode_ms": round(dec_avg, 4),
+        "encode_ms_median": round(enc_ms[len(enc_ms) // 2], 4),
+        "decode_ms_median": round(dec_ms[len(dec_ms) // 2], 4),
         "encode_roofline_frac": round(ab["encode"] / (enc_avg * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
         "decode_roofline_frac": round(ab["decode"] / (dec_avg * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
         "compression_ratio_payload": round(kv_bytes / payload, 3),

@@ -849,6 +849,7 @@ struct EncodeArgs {
     int32_t cap;
     int32_t *lengths;       // [sub][row][channel]
     int32_t *status;        // may be null
+    int64_t *tile_sums;     // SLOTS, one block per tile of kSlotTile streams: stored bytes per tile, or null
     const float *key_bins, *value_bins;     // float32 [L] each, or null when the levels are not known
     int64_t L;
     StreamGrid sg;
@@ -978,6 +979,21 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
     const int len = enc.finish();
     a.lengths[stream] = len;
     if (len > a.cap && a.status) atomicOr(a.status, 1);
+    if (SLOTS && a.tile_sums) {
+        // every lane of the block is active here (the host asks for tile sums only when a block
+        // is exactly one tile): bytes the block's streams occupy in the payload
+        __shared__ int32_t wave_sums[BS / 64];
+        int32_t v = len < a.cap ? len : a.cap;
+#pragma unroll
+        for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
+        if ((tid & 63) == 0) wave_sums[tid >> 6] = v;
+        __syncthreads();
+        if (tid == 0) {
+            int64_t total = 0;
+            for (int w = 0; w < BS / 64; ++w) total += wave_sums[w];
+            a.tile_sums[blockIdx.x] = total;
+        }
+    }
 }
 
 // ---- decoder (dec_new.cu:35-71, 248-302) -------------------------------------------
@@ -1364,17 +1380,35 @@ __global__ __launch_bounds__(kScanThreads) void scan_tile_sums_kernel(
     if (threadIdx.x == 0) sums[blockIdx.x] = total;
 }
 
+// In place, one block: every thread owns a contiguous run of the sums, adds it up, the block
+// scans the 256 run totals, and every thread rewrites its run as exclusive running sums.
+// Runs are handled 16 values at a time from registers so that the loads are in flight together.
 __global__ __launch_bounds__(kScanThreads) void scan_sums_kernel(int64_t *sums, int64_t ntiles)
 {
     __shared__ int64_t lds[kScanThreads];
-    int64_t carry = 0;
-    for (int64_t base = 0; base < ntiles; base += kScanThreads) {
-        const int64_t i = base + threadIdx.x;
-        const int64_t v = i < ntiles ? sums[i] : 0;
-        int64_t total;
-        const int64_t ex = block_exclusive_scan(v, lds, total);
-        if (i < ntiles) sums[i] = carry + ex;
-        carry += total;
+    constexpr int kBatch = 16;
+    const int64_t per = (ntiles + kScanThreads - 1) / kScanThreads;
+    const int64_t lo = (int64_t)threadIdx.x * per;
+    const int64_t hi = lo + per < ntiles ? lo + per : ntiles;
+    int64_t mine = 0;
+    for (int64_t i0 = lo; i0 < hi; i0 += kBatch) {
+        int64_t v[kBatch];
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j) v[j] = i0 + j < hi ? sums[i0 + j] : 0;
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j) mine += v[j];
+    }
+    int64_t total;
+    int64_t run = block_exclusive_scan(mine, lds, total);
+    for (int64_t i0 = lo; i0 < hi; i0 += kBatch) {
+        int64_t v[kBatch];
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j) v[j] = i0 + j < hi ? sums[i0 + j] : 0;
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j) {
+            if (i0 + j < hi) sums[i0 + j] = run;
+            run += v[j];
+        }
     }
 }
 
@@ -1413,19 +1447,42 @@ __global__ __launch_bounds__(kScanThreads) void scan_apply_kernel(
 constexpr int kCompactStreams = 256;
 constexpr int kCompactTile = 16384;
 
+// SCAN: the offsets are not known yet; `offsets` is written here from the streams' lengths and
+// the exclusive running sum of the tiles' byte counts (tile_base), instead of being read.
+template <bool SCAN>
 __global__ __launch_bounds__(256) void compact_streams_kernel(
-    const uint8_t *__restrict__ slots, int32_t cap, const int64_t *__restrict__ offsets,
+    const uint8_t *__restrict__ slots, int32_t cap, int64_t *__restrict__ offsets,
+    const int32_t *__restrict__ lengths, const int64_t *__restrict__ tile_base,
     int64_t nstreams, uint8_t *__restrict__ payload, int64_t payload_cap, int32_t skew, int32_t *status)
 {
     __shared__ int32_t rel[kCompactStreams + 1];       // stream offsets relative to the block's first byte
-    __shared__ uint32_t buf[kCompactTile / 4];
+    __shared__ __align__(16) uint32_t buf[kCompactTile / 4];
     const int tid = threadIdx.x;
     const int64_t sbase = (int64_t)blockIdx.x * kCompactStreams;
     const int count = (nstreams - sbase < kCompactStreams) ? (int)(nstreams - sbase) : kCompactStreams;
-    const int64_t o0 = offsets[sbase];
-    for (int i = tid; i <= kCompactStreams; i += 256)
-        rel[i] = (int32_t)(offsets[sbase + (i < count ? i : count)] - o0);
-    __syncthreads();
+    int64_t o0;
+    if (SCAN) {
+        int32_t mine = 0;
+        if (tid < count) {
+            mine = lengths[sbase + tid];
+            mine = mine < 0 ? 0 : (mine > cap ? cap : mine);
+        }
+        int64_t *lds = reinterpret_cast<int64_t *>(buf);       // kScanThreads values; buf is free until the copy
+        int64_t total64;
+        const int32_t before = (int32_t)block_exclusive_scan(mine, lds, total64);
+        o0 = tile_base[blockIdx.x];
+        rel[tid] = before;
+        if (tid == 0) rel[kCompactStreams] = (int32_t)total64;
+        if (tid < count) offsets[sbase + tid] = o0 + before;
+        if (sbase + count == nstreams && tid == 0) offsets[nstreams] = o0 + total64;
+        __syncthreads();
+        // threads past the last stream carry the total, like the padding of the other form
+    } else {
+        o0 = offsets[sbase];
+        for (int i = tid; i <= kCompactStreams; i += 256)
+            rel[i] = (int32_t)(offsets[sbase + (i < count ? i : count)] - o0);
+        __syncthreads();
+    }
     const int total = rel[count];
     if (o0 + total > payload_cap) {                    // never write past the caller's buffer
         if (tid == 0 && status) atomicOr(status, 2);
@@ -1847,6 +1904,7 @@ size_t cg_encode_kv_workspace(int64_t L, int64_t T, int64_t C, int64_t chunk_tok
     size_t total = align_up((size_t)nstreams * kSub, 256);        // symbols: a 256-token slot per stream
     total += (size_t)ceil_div(nstreams, kSlotTile) * kSlotTile * kStreamCap;   // encoder scratch: whole tiles of slots
     total += cg_scan_workspace(nstreams);
+    total += align_up((size_t)ceil_div(nstreams, kSlotTile) * sizeof(int64_t), 256);   // bytes per tile of streams
     return total;
 }
 
@@ -1878,6 +1936,8 @@ int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int
     uint8_t *scratch = ws;     // kStreamCap bytes per stream, in tiles of kSlotTile word-interleaved streams
     ws += (size_t)ceil_div(nstreams, kSlotTile) * kSlotTile * kStreamCap;
     void *scan_scratch = ws;
+    ws += cg_scan_workspace(nstreams);
+    int64_t *tile_sums = reinterpret_cast<int64_t *>(ws);
     uint16_t *tables = reinterpret_cast<uint16_t *>(cdf);
 
     clear_status_kernel<<<1, 1, 0, s>>>(status);
@@ -1899,6 +1959,10 @@ int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int
     if (int rc = make_grid(rows, C, T, chunk_tokens, nsub, block, a.sg, nblocks)) return rc;
     const size_t shmem = (size_t)lp * block * sizeof(uint16_t);
     const dim3 grid((unsigned)nblocks), blk(block);
+    // when every encoder block is exactly one tile of the scratch, the blocks leave their byte
+    // counts behind and the compaction computes the stream offsets itself
+    const bool fused_scan = block == kSlotTile && C % kSlotTile == 0;
+    a.tile_sums = fused_scan ? tile_sums : nullptr;
 
     const bool packed = kv_vectorizable(kv, D, C, sl, skv, st, sh) && C % 8 == 0;
     if (delta_group > 0 && !packed)
@@ -1928,12 +1992,18 @@ int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int
     }
     if (int rc = check_launch("encode_kv")) return rc;
 
-    if (int rc = launch_scan(lengths, nstreams, kStreamCap, offsets, scan_scratch, s)) return rc;
     const int64_t cblocks = ceil_div(nstreams, kCompactStreams);
     if (cblocks > INT_MAX) return fail(CG_ERR_ARG, "encode_kv: too many streams");
-    compact_streams_kernel<<<dim3((unsigned)cblocks), dim3(256), 0, s>>>(
-        scratch, kStreamCap, offsets, nstreams, payload, payload_cap,
-        (int32_t)(reinterpret_cast<uintptr_t>(payload) & 3u), status);
+    const int32_t skew = (int32_t)(reinterpret_cast<uintptr_t>(payload) & 3u);
+    if (fused_scan) {
+        scan_sums_kernel<<<dim3(1), dim3(kScanThreads), 0, s>>>(tile_sums, cblocks);
+        compact_streams_kernel<true><<<dim3((unsigned)cblocks), dim3(256), 0, s>>>(
+            scratch, kStreamCap, offsets, lengths, tile_sums, nstreams, payload, payload_cap, skew, status);
+    } else {
+        if (int rc = launch_scan(lengths, nstreams, kStreamCap, offsets, scan_scratch, s)) return rc;
+        compact_streams_kernel<false><<<dim3((unsigned)cblocks), dim3(256), 0, s>>>(
+            scratch, kStreamCap, offsets, nullptr, nullptr, nstreams, payload, payload_cap, skew, status);
+    }
     return check_launch("compact");
 }
 

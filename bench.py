@@ -21,9 +21,9 @@ HBM_PEAK_GBPS = 8000.0
 
 # HBM bytes per launch of decode_streams_kernel measured with rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE (two runs, each scaled by what the same counter reads for a plain conversion
-# kernel of known size: x2.000 and x1.000): 346.1 MB read + 1073.7 MB written.  A profile
+# kernel of known size: x2.000 and x1.000): 310.4 MB read + 1073.7 MB written.  A profile
 # measurement of this workload, not something this script can observe while it runs.
-MEASURED_DECODE_TRAFFIC_BYTES = {"config2": 1419.8e6}
+MEASURED_DECODE_TRAFFIC_BYTES = {"config2": 1384.1e6}
 
 WORKLOADS = {
     # name: (layers, tokens, heads, head_size, chunk_tokens, model name for the bins table, seed)

@@ -1746,6 +1746,7 @@ void launch_decode_kv_log2(const DecodeArgs &a, dim3 grid, size_t shmem, hipStre
 {
     const dim3 blk(BS);
     switch (a.lp) {
+    case 9: decode_streams_kernel<BS, 3, SRC_OFFSETS, OUT><<<grid, blk, shmem, stream>>>(a); break;
     case 17: decode_streams_kernel<BS, 4, SRC_OFFSETS, OUT><<<grid, blk, shmem, stream>>>(a); break;
     case 33: decode_streams_kernel<BS, 5, SRC_OFFSETS, OUT><<<grid, blk, shmem, stream>>>(a); break;
     case 65: decode_streams_kernel<BS, 6, SRC_OFFSETS, OUT><<<grid, blk, shmem, stream>>>(a); break;

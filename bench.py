@@ -161,6 +161,8 @@ def main():
     ap.add_argument("--workload", default="config2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-tokens", type=int, default=8192)
+    ap.add_argument("--fmt", default="vllm", choices=["vllm", "huggingface"],
+                    help="layout of the KV tensor: [L,2,T,H,D] (vllm, the metric's layout) or [L,2,H,T,D]")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one plain device copy of the KV tensor (calibrates rocprofv3 byte counters)")
     args = ap.parse_args()
@@ -183,19 +185,22 @@ def main():
     torch.cuda.set_device(dev)
     kbins, vbins = bins_for(args.workload, model, L)
     kv = make_kv(L, T, H, D, seed=seed, device=dev)
+    fmt = args.fmt
+    if fmt == "huggingface":
+        kv = kv.permute(0, 1, 3, 2, 4).contiguous()
     kb, vb = kbins.to(dev), vbins.to(dev)
     max_bins = int(max(kbins.max(), vbins.max()))
 
     workspace = torch.empty(codec.encode_workspace_bytes(L, T, C, chunk), dtype=torch.uint8, device=dev)
-    enc = codec.encode_kv(kv, kb, vb, chunk_tokens=chunk, max_bins=max_bins, workspace=workspace)
+    enc = codec.encode_kv(kv, kb, vb, chunk_tokens=chunk, max_bins=max_bins, workspace=workspace, fmt=fmt)
     enc.check()
-    out = torch.empty((L, 2, T, H, D), dtype=torch.float16, device=dev)
+    out = torch.empty_like(kv)
 
     def encode():
-        codec.encode_kv(kv, kb, vb, chunk_tokens=chunk, max_bins=max_bins, workspace=workspace, out=enc)
+        codec.encode_kv(kv, kb, vb, chunk_tokens=chunk, max_bins=max_bins, workspace=workspace, out=enc, fmt=fmt)
 
     def decode():
-        codec.decode_encoded(enc, kb, vb, fmt="vllm", out=out)
+        codec.decode_encoded(enc, kb, vb, fmt=fmt, out=out)
 
     for _ in range(args.warmup):
         encode()
@@ -238,8 +243,11 @@ def main():
     maxq = torch.stack([kb, vb], dim=1).div(2, rounding_mode="floor").sub(1)[:, :, None, None]
     verified = True
     for l0 in range(0, L, 8):
-        x = kv[l0:l0 + 8].reshape(-1, 2, T, C).float()
-        y = out[l0:l0 + 8].reshape(-1, 2, T, C).float()
+        xs, ys = kv[l0:l0 + 8], out[l0:l0 + 8]
+        if fmt == "huggingface":
+            xs, ys = xs.permute(0, 1, 3, 2, 4), ys.permute(0, 1, 3, 2, 4)
+        x = xs.reshape(-1, 2, T, C).float()
+        y = ys.reshape(-1, 2, T, C).float()
         step = x.abs().amax(dim=-1, keepdim=True) / maxq[l0:l0 + 8]
         verified = verified and bool(((x - y).abs() <= 0.52 * step).all())
         del x, y
@@ -259,7 +267,8 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": "%s: %d layers x {K,V} x %d tokens x %d heads x %d, fp16, one table per %d tokens, "
-                        "AR(1) rho=0.9 lognormal-channel generator seed %d" % (args.workload, L, T, H, D, chunk, seed),
+                        "AR(1) rho=0.9 lognormal-channel generator seed %d%s"
+                        % (args.workload, L, T, H, D, chunk, seed, "" if fmt == "vllm" else ", layout [L,2,H,T,D]"),
             "value_is": "fp16 KV bytes encoded plus decoded per second of a full encode+decode step",
             "kv_bytes": kv_bytes,
             "streams": nstreams,
@@ -290,19 +299,21 @@ def main():
     }
     if chunk > 256:
         # streaming case: latency of decoding one chunk on its own
-        one = codec.encode_kv(kv[:, :, :chunk], kb, vb, chunk_tokens=chunk, max_bins=max_bins)
-        one_out = torch.empty((L, 2, chunk, H, D), dtype=torch.float16, device=dev)
+        tdim = 2 if fmt == "vllm" else 3
+        one = codec.encode_kv(kv.narrow(tdim, 0, chunk), kb, vb, chunk_tokens=chunk, max_bins=max_bins, fmt=fmt)
+        one_out = torch.empty_like(kv.narrow(tdim, 0, chunk))
         for _ in range(3):
-            codec.decode_encoded(one, kb, vb, fmt="vllm", out=one_out)
+            codec.decode_encoded(one, kb, vb, fmt=fmt, out=one_out)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for _ in range(10):
-            codec.decode_encoded(one, kb, vb, fmt="vllm", out=one_out)
+            codec.decode_encoded(one, kb, vb, fmt=fmt, out=one_out)
         e1.record()
         torch.cuda.synchronize()
         result["decode_ms_per_%d_token_chunk" % chunk] = round(e0.elapsed_time(e1) / 10, 4)
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(kv[:, :, :args.cpu_sample_tokens].cpu(), kbins, vbins, chunk,
+        kv_vllm = kv if fmt == "vllm" else kv.permute(0, 1, 3, 2, 4)
+        result["cpu_baseline"] = cpu_baseline(kv_vllm[:, :, :args.cpu_sample_tokens].cpu(), kbins, vbins, chunk,
                                               args.cpu_sample_tokens)
     print(json.dumps(result))
 

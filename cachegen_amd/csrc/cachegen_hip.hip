@@ -1019,7 +1019,7 @@ struct BitReader {
     const uint8_t *base;     // the aligned word holding the stream's first byte
     uint32_t last;           // byte offset from `base` of the last word that may be read
     uint32_t pos;            // byte offset from `base` of the next word to fetch
-    uint32_t hi, lo;         // the next `avail` bits of the stream, left-aligned, zeros below
+    uint64_t win;            // the next `avail` bits of the stream, left-aligned, zeros below
     int avail;
     uint32_t nextw;          // the word after the window, as loaded
 
@@ -1034,6 +1034,9 @@ struct BitReader {
     // whose last readable word is at byte offset `last_word`; returns the first 32 bits
     __device__ __forceinline__ uint32_t start(const uint8_t *window, int64_t last_word, int64_t begin)
     {
+        // a start outside the buffer (offsets that are not running sums of stream lengths) is
+        // moved inside it: such a stream decodes to garbage, never to a read out of bounds
+        begin = begin < 0 ? 0 : (begin > last_word ? last_word : begin);
         const uint32_t skip = (uint32_t)begin & 3u;
         const int64_t first_word = begin - skip;
         base = window + first_word;
@@ -1046,8 +1049,7 @@ struct BitReader {
         const uint32_t s = skip * 8u;
         const uint64_t head = (((uint64_t)b0 << 32) | b1) << s;
         const uint64_t rest = (((uint64_t)b1 << 32) | b2) << s;
-        hi = (uint32_t)(rest >> 32);
-        lo = (uint32_t)rest;
+        win = rest;
         avail = 64 - (int)s;
         return (uint32_t)(head >> 32);
     }
@@ -1055,10 +1057,8 @@ struct BitReader {
     // off = (off << n) | next n bits, 0 <= n <= 31 and n <= avail
     __device__ __forceinline__ uint32_t shift_in(uint32_t off, int n)
     {
-        off = (uint32_t)(((((uint64_t)off) << 32) | hi) >> (32 - n));
-        const uint64_t w = ((((uint64_t)hi) << 32) | lo) << n;
-        hi = (uint32_t)(w >> 32);
-        lo = (uint32_t)w;
+        off = (off << n) | __builtin_amdgcn_ubfe((uint32_t)(win >> 32), (uint32_t)(32 - n), (uint32_t)n);   // n = 0 extracts nothing
+        win <<= n;
         avail -= n;
         return off;
     }
@@ -1067,9 +1067,7 @@ struct BitReader {
     __device__ __forceinline__ void top_up()
     {
         if (avail <= 32) {                      // the low word is empty
-            const uint64_t w = (((uint64_t)__builtin_bswap32(nextw)) << 32) >> (avail & 63);
-            hi |= (uint32_t)(w >> 32);
-            lo = (uint32_t)w;
+            win |= (((uint64_t)__builtin_bswap32(nextw)) << 32) >> (avail & 63);
             avail += 32;
             nextw = raw();
         }

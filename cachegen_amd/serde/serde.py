@@ -1,5 +1,6 @@
 """Serializer / Deserializer plug-in interface
-(LMCache/lmcache/storage_backend/serde/serde.py:9-63 in the reference)."""
+(LMCache/lmcache/storage_backend/serde/serde.py:9-63 in the reference): a serializer turns a
+chunk tensor into bytes, a deserializer turns them back."""
 import abc
 import logging
 import time
@@ -12,40 +13,46 @@ logger = logging.getLogger("cachegen_amd")
 class Serializer(metaclass=abc.ABCMeta):
     @abc.abstractmethod
     def to_bytes(self, t: torch.Tensor) -> bytes:
-        """Serialize a tensor (data and metadata) to bytes."""
+        """The tensor, data and whatever is needed to rebuild it, as bytes."""
         raise NotImplementedError
 
 
 class Deserializer(metaclass=abc.ABCMeta):
     @abc.abstractmethod
     def from_bytes(self, bs: bytes) -> torch.Tensor:
-        """Rebuild the tensor from `to_bytes` output."""
+        """The tensor that `to_bytes` was given (or its lossy reconstruction)."""
         raise NotImplementedError
 
 
-class SerializerDebugWrapper(Serializer):
-    def __init__(self, s: Serializer):
-        self.s = s
+class _Timed:
+    """Wraps a serde object: the one interface call is timed into the debug log, everything
+    else the wrapped object offers passes through."""
 
-    def to_bytes(self, t: torch.Tensor) -> bytes:
-        start = time.perf_counter()
-        bs = self.s.to_bytes(t)
-        logger.debug("Serialization took %.2f seconds", time.perf_counter() - start)
-        return bs
+    def __init__(self, inner, what):
+        self._inner = inner
+        self._what = what
 
-    def __getattr__(self, name):           # whatever else the wrapped serializer offers
-        return getattr(self.s, name)
-
-
-class DeserializerDebugWrapper(Deserializer):
-    def __init__(self, d: Deserializer):
-        self.d = d
-
-    def from_bytes(self, bs: bytes) -> torch.Tensor:
-        start = time.perf_counter()
-        ret = self.d.from_bytes(bs)
-        logger.debug("Deserialization took %.2f ms", (time.perf_counter() - start) * 1000)
+    def _run(self, fn, arg):
+        t0 = time.perf_counter()
+        ret = fn(arg)
+        logger.debug("%s took %.2f ms", self._what, (time.perf_counter() - t0) * 1e3)
         return ret
 
     def __getattr__(self, name):
-        return getattr(self.d, name)
+        return getattr(self._inner, name)
+
+
+class SerializerDebugWrapper(_Timed, Serializer):
+    def __init__(self, s: Serializer):
+        _Timed.__init__(self, s, "Serialization")
+
+    def to_bytes(self, t: torch.Tensor) -> bytes:
+        return self._run(self._inner.to_bytes, t)
+
+
+class DeserializerDebugWrapper(_Timed, Deserializer):
+    def __init__(self, d: Deserializer):
+        _Timed.__init__(self, d, "Deserialization")
+
+    def from_bytes(self, bs: bytes) -> torch.Tensor:
+        return self._run(self._inner.from_bytes, bs)

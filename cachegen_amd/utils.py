@@ -1,7 +1,6 @@
-"""Key and type definitions shared by the cache engine and its backends
+"""Key and type definitions shared by the cache engine and its stores
 (LMCache/lmcache/utils.py:8-31 in the reference)."""
-from dataclasses import dataclass
-from typing import Tuple
+from typing import NamedTuple, Tuple
 
 import torch
 
@@ -10,8 +9,9 @@ import torch
 KVCache = Tuple[Tuple[torch.Tensor, torch.Tensor], ...]
 
 
-@dataclass(frozen=True)
-class CacheEngineKey:
+class CacheEngineKey(NamedTuple):
+    """What a stored chunk is filed under.  Its string form, the five fields joined by "@",
+    is the key on the remote side, so a model name must not contain "@"."""
     fmt: str
     model_name: str
     world_size: int
@@ -19,11 +19,12 @@ class CacheEngineKey:
     chunk_hash: str
 
     def to_string(self) -> str:
-        return f"{self.fmt}@{self.model_name}@{self.world_size}@{self.worker_id}@{self.chunk_hash}"
+        return "@".join(str(field) for field in self)
 
-    @staticmethod
-    def from_string(s: str) -> "CacheEngineKey":
-        parts = s.split("@")
-        if len(parts) != 5:
+    @classmethod
+    def from_string(cls, s: str) -> "CacheEngineKey":
+        fields = s.split("@")
+        if len(fields) != 5:
             raise ValueError(f"Invalid key string: {s}")
-        return CacheEngineKey(parts[0], parts[1], int(parts[2]), int(parts[3]), parts[4])
+        fmt, model_name, world_size, worker_id, chunk_hash = fields
+        return cls(fmt, model_name, int(world_size), int(worker_id), chunk_hash)

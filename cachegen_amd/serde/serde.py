@@ -46,6 +46,10 @@ class SerializerDebugWrapper(_Timed, Serializer):
     def __init__(self, s: Serializer):
         _Timed.__init__(self, s, "Serialization")
 
+    @property
+    def s(self) -> Serializer:          # the wrapped serializer, under the reference's attribute name
+        return self._inner
+
     def to_bytes(self, t: torch.Tensor) -> bytes:
         return self._run(self._inner.to_bytes, t)
 
@@ -53,6 +57,10 @@ class SerializerDebugWrapper(_Timed, Serializer):
 class DeserializerDebugWrapper(_Timed, Deserializer):
     def __init__(self, d: Deserializer):
         _Timed.__init__(self, d, "Deserialization")
+
+    @property
+    def d(self) -> Deserializer:
+        return self._inner
 
     def from_bytes(self, bs: bytes) -> torch.Tensor:
         return self._run(self._inner.from_bytes, bs)

@@ -1,0 +1,113 @@
+// Part of the CacheGen KV codec library for MI355X (gfx950); included by cachegen_hip.hip, which
+// is the one translation unit.  Error reporting, 16-bit float conversions and small device helpers shared by every kernel.
+//
+// Paths in the comments are relative to LMCache/ in the reference tree:
+//   enc_new.cu = third_party/torchac_cuda/torchac_kernel_enc_new.cu
+//   dec_new.cu = third_party/torchac_cuda/torchac_kernel_dec_new.cu
+//   cal_cdf.cu = third_party/torchac_cuda/cal_cdf.cu
+//   encoder.py = lmcache/storage_backend/serde/cachegen_encoder.py
+//   decoder.py = lmcache/storage_backend/serde/cachegen_decoder.py
+#pragma once
+
+namespace {
+
+// ------------------------------------------------------------------------------------
+// host-side helpers
+// ------------------------------------------------------------------------------------
+thread_local char g_error[512] = "";
+
+int fail(int code, const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int check_launch(const char *what)
+{
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(CG_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+    return CG_OK;
+}
+
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+inline bool aligned_to(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+constexpr int kSub = CG_MAX_TOKENS_PER_STREAM;   // tokens per stream (cachegen_basics.py:8)
+constexpr int kStreamCap = 256;                  // bytes kept per stream in the fused path
+
+// Token geometry shared by the stream kernels: chunk k covers tokens
+// [k*S, min((k+1)*S, T)), and is cut every 256 tokens (encoder.py:279-292).
+struct TokenGeom {
+    int64_t T;        // tokens in the tensor
+    int64_t S;        // tokens per chunk (one table per chunk)
+    int32_t nsc;      // sub-chunks in a full chunk = ceil(S / 256)
+};
+
+__host__ __device__ inline void sub_range(const TokenGeom &g, int64_t sub, int64_t &chunk,
+                                          int64_t &t0, int &n)
+{
+    chunk = sub / g.nsc;
+    const int64_t j = sub - chunk * g.nsc;
+    t0 = chunk * g.S + j * kSub;
+    int64_t tend = (chunk + 1) * g.S;
+    if (tend > g.T) tend = g.T;
+    const int64_t left = tend - t0;
+    n = left < kSub ? (int)left : kSub;
+}
+
+// ------------------------------------------------------------------------------------
+// device helpers
+// ------------------------------------------------------------------------------------
+__device__ __forceinline__ float f16_bits_to_float(uint32_t h)
+{
+    _Float16 v;
+    uint16_t b = (uint16_t)h;
+    __builtin_memcpy(&v, &b, 2);
+    return (float)v;
+}
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t h) { return __uint_as_float(h << 16); }
+
+template <int DT>
+__device__ __forceinline__ float load16f(uint32_t bits)
+{
+    return DT == CG_DT_BF16 ? bf16_bits_to_float(bits) : f16_bits_to_float(bits);
+}
+
+__device__ __forceinline__ uint32_t float_to_f16_bits(float f)
+{
+    _Float16 v = (_Float16)f;      // v_cvt_f16_f32, round to nearest even
+    uint16_t b;
+    __builtin_memcpy(&b, &v, 2);
+    return b;
+}
+__device__ __forceinline__ uint32_t float_to_bf16_bits(float f)
+{
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (u >> 16) | 0x40u;
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+template <int DT>
+__device__ __forceinline__ uint32_t store16f(float f)
+{
+    return DT == CG_DT_BF16 ? float_to_bf16_bits(f) : float_to_f16_bits(f);
+}
+
+// 24-bit multiply, low 32 bits of the product, as an unsigned value (HIP's __umul24 returns
+// int, which would turn a following >> into an arithmetic shift).
+__device__ __forceinline__ uint32_t mul24(uint32_t a, uint32_t b) { return (uint32_t)__umul24(a, b); }
+
+// floor(span * c / 2^16), the `(span * c) >> precision` of enc_new.cu:272-273 and
+// dec_new.cu:280-281, on the full-rate 24-bit multiplier from the span's halves
+// (sh = span >> 16, sl = span & 0xffff): span*c = sh*c*2^16 + sl*c.  Valid for every span
+// below 2^32 and every c up to and including 2^16 (where it returns the span).
+__device__ __forceinline__ uint32_t scale_span(uint32_t sh, uint32_t sl, uint32_t c)
+{
+    return mul24(sh, c) + (mul24(sl, c) >> 16);
+}
+
+}  // namespace

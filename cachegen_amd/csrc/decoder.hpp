@@ -1,0 +1,353 @@
+// Part of the CacheGen KV codec library for MI355X (gfx950); included by cachegen_hip.hip, which
+// is the one translation unit.  Range decoder: bit reader, symbol search, fused dequantisation, decode_streams_kernel.
+//
+// Paths in the comments are relative to LMCache/ in the reference tree:
+//   enc_new.cu = third_party/torchac_cuda/torchac_kernel_enc_new.cu
+//   dec_new.cu = third_party/torchac_cuda/torchac_kernel_dec_new.cu
+//   cal_cdf.cu = third_party/torchac_cuda/cal_cdf.cu
+//   encoder.py = lmcache/storage_backend/serde/cachegen_encoder.py
+//   decoder.py = lmcache/storage_backend/serde/cachegen_decoder.py
+#pragma once
+
+namespace {
+
+// ---- decoder (dec_new.cu:35-71, 248-302) -------------------------------------------
+// The decoder tracks off = value - low, which every renormalisation step maps to
+// 2*off + next bit (E1/E2 and E3 alike), and finds the symbol as the largest m with
+// T(m) = floor(span*cdf[m] / 2^16) <= off; that is the same m as the reference's search
+// of count = ((value-low+1)*2^16 - 1) / span in a strictly increasing table, without the
+// 64-bit divide.  For tables of 2^k symbols the search probes with the lower bound
+// (span >> 16) * cdf[m] <= T(m) (one multiply), which can only overshoot, and the result
+// is then walked back while the exact T(m) exceeds off (almost never).
+//
+// The stream is read through aligned big-endian words into a 64-bit window of unread bits.
+// Every lane of a wavefront runs the refill code whenever one lane needs it, so the window
+// is topped up at fixed points, once per two symbols, instead of whenever a lane runs dry:
+// after a top-up it holds more than 32 bits, a symbol of a table without zero-width entries
+// consumes at most 18 (the span stays above 2^30), and the one case left (fewer than 18 bits
+// before the second symbol of a pair) takes an extra top-up.
+// Bits past the end of a stream are whatever follows it in memory instead of the reference's
+// zeros (dec_new.cu:223-233): the coder's two closing bits place the code value inside
+// the final interval for every continuation, so the n symbols that were encoded decode
+// identically.  Word loads are clamped to the last word of the byte buffer.
+struct BitReader {
+    const uint8_t *base;     // the aligned word holding the stream's first byte
+    uint32_t last;           // byte offset from `base` of the last word that may be read
+    uint32_t pos;            // byte offset from `base` of the next word to fetch
+    uint64_t win;            // the next `avail` bits of the stream, left-aligned, zeros below
+    int avail;
+    uint32_t nextw;          // the word after the window, as loaded
+
+    __device__ __forceinline__ uint32_t raw()
+    {
+        const uint32_t at = pos < last ? pos : last;
+        pos += 4;
+        return *reinterpret_cast<const uint32_t *>(base + at);
+    }
+
+    // position on the stream that begins `begin` bytes after the 4-byte aligned `window`,
+    // whose last readable word is at byte offset `last_word`; returns the first 32 bits
+    __device__ __forceinline__ uint32_t start(const uint8_t *window, int64_t last_word, int64_t begin)
+    {
+        // a start outside the buffer (offsets that are not running sums of stream lengths) is
+        // moved inside it: such a stream decodes to garbage, never to a read out of bounds
+        begin = begin < 0 ? 0 : (begin > last_word ? last_word : begin);
+        const uint32_t skip = (uint32_t)begin & 3u;
+        const int64_t first_word = begin - skip;
+        base = window + first_word;
+        const int64_t room = last_word - first_word;
+        last = room < 0 ? 0u : (room > 0xFFFFFFF0ll ? 0xFFFFFFF0u : (uint32_t)room);
+        pos = 0;
+        const uint32_t b0 = __builtin_bswap32(raw()), b1 = __builtin_bswap32(raw());
+        const uint32_t b2 = __builtin_bswap32(raw());
+        nextw = raw();
+        const uint32_t s = skip * 8u;
+        const uint64_t head = (((uint64_t)b0 << 32) | b1) << s;
+        const uint64_t rest = (((uint64_t)b1 << 32) | b2) << s;
+        win = rest;
+        avail = 64 - (int)s;
+        return (uint32_t)(head >> 32);
+    }
+
+    // off = (off << n) | next n bits, 0 <= n <= 31 and n <= avail
+    __device__ __forceinline__ uint32_t shift_in(uint32_t off, int n)
+    {
+        off = (off << n) | __builtin_amdgcn_ubfe((uint32_t)(win >> 32), (uint32_t)(32 - n), (uint32_t)n);   // n = 0 extracts nothing
+        win <<= n;
+        avail -= n;
+        return off;
+    }
+
+    // brings the window to more than 32 bits
+    __device__ __forceinline__ void top_up()
+    {
+        if (avail <= 32) {                      // the low word is empty
+            win |= (((uint64_t)__builtin_bswap32(nextw)) << 32) >> (avail & 63);
+            avail += 32;
+            nextw = raw();
+        }
+    }
+};
+
+enum { SRC_OFFSETS = 0, SRC_PREFIX = 1, SRC_PADDED = 2 };
+enum { OUT_SYMBOLS = 0, OUT_F16 = 1, OUT_BF16 = 2 };
+
+struct DecodeArgs {
+    const uint16_t *cdf;
+    int32_t lp;
+    const uint8_t *bytes;       // payload or padded buffer, rounded down to a 4-byte boundary
+    uint32_t bytes_skew;        // bytes dropped by that rounding (0..3)
+    int64_t last_word;          // byte offset from `bytes` of the last readable word
+    const int64_t *offsets;     // SRC_OFFSETS: exclusive sums [nstreams+1]; SRC_PREFIX: inclusive sums
+    int64_t p0, p1;             // SRC_PADDED strides
+    // OUT_SYMBOLS: out[row*o0 + token*o1 + channel*o2] uint8
+    uint8_t *out_sym;
+    int64_t o0, o1, o2;
+    // OUT_F16 / OUT_BF16: dequantised KV, out[l*ol + kv*okv + token*ot + head*oh + dim]
+    uint16_t *out_kv;
+    int64_t ol, okv, ot, oh;
+    int64_t L;
+    int32_t D;
+    const uint16_t *maxima;     // [2, L, T]
+    int32_t max_dt;
+    int32_t delta_group;        // > 0: rows that are not the first of their group hold deltas
+    const float *key_bins, *value_bins;
+    StreamGrid sg;
+};
+
+// Tables in LDS for the decoder: entry e of lane c's column is the 16-bit word at byte
+// e * kRow + 2 * c.  When the kernel dequantises, every row carries one float behind the
+// lanes' entries: (e - C) / C, the quotient of symbol e (decoder.py:28-31).
+template <int BS, int OUT>
+struct DecodeLayout {
+    static constexpr int kRow = OUT == OUT_SYMBOLS ? 2 * BS : 2 * BS + 4;
+    static constexpr int kQuot = 2 * BS;          // byte offset of the quotient inside a row
+};
+
+typedef __attribute__((address_space(3))) const uint16_t lds_u16;
+typedef __attribute__((address_space(3))) const float lds_f32;
+typedef __attribute__((address_space(3))) const char lds_char;
+
+__device__ __forceinline__ uint32_t lds_entry(lds_char *p, int byte_offset)
+{
+    return *(lds_u16 *)(p + byte_offset);
+}
+
+// float32 -> bfloat16 bits, round to nearest even, for anything but a NaN
+__device__ __forceinline__ uint32_t float_to_bf16_bits_no_nan(float f)
+{
+    uint32_t u = __float_as_uint(f);
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+
+struct DecodeLane {
+    BitReader rd;
+    uint32_t off, low, span;
+    lds_char *colp;            // this lane's entry 0
+    int lutoff;                // from an entry of this lane to its row's quotient
+    uint8_t *osym;
+    uint16_t *okv;
+    float anchor;              // reconstructed anchor row value (delta mode)
+    int phase;                 // position of the token inside its group (delta mode)
+};
+
+// One symbol.  SKIP: how many of the search's first probes are left out because the row's
+// alphabet fits the lower 2^(LOG2-SKIP) entries.  SAFE: the last table entry may be decoded
+// (its upper bound 2^16 is substituted, dec_new.cu:278) and values may be NaN.
+template <int BS, int LOG2, int OUT, int SKIP, bool SAFE>
+__device__ __forceinline__ void decode_symbol(const DecodeArgs &a, DecodeLane &s, int lp, int nsteps,
+                                              float rm, int i, bool last_symbol)
+{
+    constexpr int kRow = DecodeLayout<BS, OUT>::kRow;
+    lds_char *p = s.colp;              // entry of the decoded symbol
+    lds_char *const plast = s.colp + (lp - 2) * kRow;
+    uint32_t t_lo, width;
+    if (__builtin_expect(s.span == 0, 0)) {
+        // full range: T(m) = cdf[m] << 16, so compare table values with off >> 16
+        const uint32_t key = s.off >> 16;
+        if (LOG2 >= 0) {
+#pragma unroll
+            for (int step = ((1 << LOG2) >> 1) >> SKIP; step >= 1; step >>= 1)
+                p = (lds_entry(p, step * kRow) <= key) ? p + step * kRow : p;
+        } else {
+            int lo_i = 0, hi_i = lp - 1;
+            for (int step = 0; step < nsteps; ++step) {
+                const int mid = (lo_i + hi_i) >> 1;
+                const bool le = mid > 0 && lds_entry(s.colp, mid * kRow) <= key;
+                lo_i = le ? mid : lo_i;
+                hi_i = le ? hi_i : mid;
+            }
+            p = s.colp + lo_i * kRow;
+        }
+        const uint32_t c_lo = lds_entry(p, 0);
+        const uint32_t c_hi = (SAFE && p == plast) ? 0x10000u : lds_entry(p, kRow);
+        t_lo = c_lo << 16;
+        width = (c_hi - c_lo) << 16;
+    } else {
+        const uint32_t sh = s.span >> 16, sl = s.span & 0xFFFFu;
+        if (LOG2 >= 0) {
+            // probe with the lower bound sh * c <= T(c); it can only overshoot
+#pragma unroll
+            for (int step = ((1 << LOG2) >> 1) >> SKIP; step >= 1; step >>= 1) {
+                const uint32_t t = mul24(sh, lds_entry(p, step * kRow));
+                p = (t <= s.off) ? p + step * kRow : p;
+            }
+            t_lo = scale_span(sh, sl, lds_entry(p, 0));
+            // entry 0 is 0 (forced when the tables are staged), so this stops there at the latest
+            while (__builtin_expect(t_lo > s.off, 0)) {
+                p -= kRow;
+                t_lo = scale_span(sh, sl, lds_entry(p, 0));
+            }
+        } else {
+            int lo_i = 0, hi_i = lp - 1;
+            for (int step = 0; step < nsteps; ++step) {
+                const int mid = (lo_i + hi_i) >> 1;
+                const uint32_t t = scale_span(sh, sl, lds_entry(s.colp, mid * kRow));
+                const bool le = mid > 0 && t <= s.off;
+                lo_i = le ? mid : lo_i;
+                hi_i = le ? hi_i : mid;
+            }
+            p = s.colp + lo_i * kRow;
+            t_lo = scale_span(sh, sl, lds_entry(p, 0));
+        }
+        const uint32_t c_hi = (SAFE && p == plast) ? 0x10000u : lds_entry(p, kRow);
+        width = scale_span(sh, sl, c_hi) - t_lo;
+    }
+    if (OUT == OUT_SYMBOLS) {
+        s.osym[(int64_t)i * a.o1] = (uint8_t)((uint32_t)(p - s.colp) / (uint32_t)kRow);
+    } else {
+        const float q = *(lds_f32 *)(p + s.lutoff);
+        float v = __fmul_rn(q, rm);
+        // the product is rounded to float32 before it is rounded to 16 bits (decoder.py:28-34
+        // works in float32): keep the compiler from merging the two into one mixed-precision
+        // multiply, which rounds once and turns -0 into +0
+        asm volatile("" : "+v"(v));
+        if (SAFE && a.delta_group > 0) {             // uniform over the block
+            if (s.phase == 0) s.anchor = v;
+            else v = __fadd_rn(v, s.anchor);
+            s.phase = s.phase + 1 == a.delta_group ? 0 : s.phase + 1;
+        }
+        uint32_t bits;
+        if (OUT == OUT_BF16) bits = SAFE ? float_to_bf16_bits(v) : float_to_bf16_bits_no_nan(v);
+        else bits = float_to_f16_bits(v);
+        *s.okv = (uint16_t)bits;
+        s.okv += a.ot;
+    }
+    if (last_symbol) return;                    // no update after the last symbol
+    s.low += t_lo;
+    s.off -= t_lo;
+    const uint32_t high = s.low + width - 1u;
+    const int n1 = __builtin_clz(s.low ^ high);
+    // E3 run: positions below the first differing bit where low has 1 and high has 0, i.e.
+    // leading zeros of (~low | high) once that bit is shifted out; the run always ends
+    // inside the word because the interval is wider than one
+    const uint32_t z = ((s.low & high) | (~s.low & 0xFFFFFFFFu)) << ((n1 + 1) & 31);   // one bit-field insert
+    const int n = n1 + __builtin_clz(z);
+    s.low = (s.low << n) & 0x7FFFFFFFu;
+    s.span = width << n;
+    s.off = s.rd.shift_in(s.off, n);
+}
+
+template <int BS, int LOG2, int OUT, int SKIP, bool SAFE>
+__device__ __forceinline__ void decode_lane(const DecodeArgs &a, DecodeLane &s, int lp, int n, lds_f32 *rmp)
+{
+    int nsteps = 0;
+    if (LOG2 < 0)
+        while ((1 << nsteps) < lp - 1) ++nsteps;
+    for (int i0 = 0; i0 < n; i0 += 4, rmp += 4) {
+        // the maxima of the next four token rows (the array is padded to a multiple of four)
+        float rm[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (OUT != OUT_SYMBOLS) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) rm[j] = rmp[j];
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int i = i0 + j;
+            if (i >= n) break;
+            if ((j & 1) == 0) s.rd.top_up();
+            else if (__builtin_expect(s.rd.avail < 18, 0)) s.rd.top_up();
+            decode_symbol<BS, LOG2, OUT, SKIP, SAFE>(a, s, lp, nsteps, rm[j], i, i == n - 1);
+        }
+    }
+}
+
+// LOG2 >= 0: the table has exactly 2^LOG2 symbols (lp = 2^LOG2 + 1) and the search is
+// unrolled with immediate LDS offsets; LOG2 < 0: any lp.
+template <int BS, int LOG2, int SRC, int OUT>
+__global__ __launch_bounds__(BS) void decode_streams_kernel(DecodeArgs a)
+{
+    extern __shared__ uint32_t smem[];
+    constexpr int kRow = DecodeLayout<BS, OUT>::kRow;
+    const int tid = threadIdx.x;
+    const StreamId id = locate<BS>(a.sg);
+    const int lp = LOG2 >= 0 ? (1 << LOG2) + 1 : a.lp;
+    char *rows = reinterpret_cast<char *>(smem);
+    float *rowmax = reinterpret_cast<float *>(rows + lp * kRow);     // one per token of the sub-chunk
+    const int64_t ch0 = id.ch - tid;
+    {
+        // entry 0 of a table is 0 by construction (cal_cdf.cu:29-49 counts into hist[sym+1]);
+        // it is stored as 0 whatever the input holds so that the walk back always ends
+        const uint16_t *src = a.cdf + ((id.chunk * a.sg.rows + id.row) * a.sg.nc + ch0) * lp;
+        const int64_t nvalid = (a.sg.nc - ch0 < BS) ? (a.sg.nc - ch0) : BS;
+        const int total = (int)nvalid * lp;
+        for (int i = tid; i < total; i += BS) {
+            const int c = i / lp, e = i - c * lp;
+            *reinterpret_cast<uint16_t *>(rows + e * kRow + 2 * c) = e == 0 ? (uint16_t)0 : src[i];
+        }
+    }
+    int64_t kvi = 0, l = 0;
+    int special = 0;                   // a row maximum that is infinite or NaN
+    int nsym = lp;                     // symbols the row's alphabet can hold
+    if (OUT != OUT_SYMBOLS) {
+        kvi = id.row / a.L;
+        l = id.row - kvi * a.L;
+        const float bins = (kvi ? a.value_bins : a.key_bins)[l];
+        const float cq = floorf(bins * 0.5f) - 1.0f;
+        nsym = (cq >= 0.0f && cq < 32768.0f) ? 2 * (int)cq + 1 : lp;
+        for (int i = tid; i < lp; i += BS)
+            *reinterpret_cast<float *>(rows + i * kRow + DecodeLayout<BS, OUT>::kQuot) =
+                __fdiv_rn(__fsub_rn((float)i, cq), cq);
+        const uint16_t *mx = a.maxima + id.row * a.sg.g.T + id.t0;
+        for (int i = tid; i < id.n; i += BS) {
+            const float m = a.max_dt == CG_DT_BF16 ? load16f<CG_DT_BF16>(mx[i]) : load16f<CG_DT_F16>(mx[i]);
+            special |= (__float_as_uint(m) & 0x7FFFFFFFu) >= 0x7F800000u;
+            rowmax[i] = m;
+        }
+    }
+    special = __syncthreads_or(special);
+    if (!id.active) return;
+
+    const int64_t stream = (id.sub * a.sg.rows + id.row) * a.sg.nc + id.ch;
+    int64_t begin;
+    if (SRC == SRC_OFFSETS) begin = a.offsets[stream];
+    else if (SRC == SRC_PREFIX) begin = stream ? a.offsets[stream - 1] : 0;
+    else begin = id.row * a.p0 + id.ch * a.p1;
+
+    DecodeLane s;
+    s.off = s.rd.start(a.bytes, a.last_word, begin + a.bytes_skew);
+    s.low = 0;
+    s.span = 0;                        // span modulo 2^32: 0 is the full range (see RangeEncoder)
+    s.colp = (lds_char *)(rows + 2 * tid);
+    s.lutoff = DecodeLayout<BS, OUT>::kQuot - 2 * tid;
+    s.osym = nullptr;
+    s.okv = nullptr;
+    s.anchor = 0.0f;
+    s.phase = 0;
+    if (OUT == OUT_SYMBOLS) {
+        s.osym = a.out_sym + id.row * a.o0 + id.t0 * a.o1 + id.ch * a.o2;
+    } else {
+        const int64_t h = id.ch / a.D;
+        s.okv = a.out_kv + l * a.ol + kvi * a.okv + id.t0 * a.ot + h * a.oh + (id.ch - h * a.D);
+    }
+    lds_f32 *rmp = (lds_f32 *)rowmax;
+
+    // all three conditions are uniform over the block
+    const bool safe = OUT == OUT_SYMBOLS || LOG2 < 0 || special || a.delta_group > 0 || nsym > lp - 2;
+    if (safe) decode_lane<BS, LOG2, OUT, 0, true>(a, s, lp, id.n, rmp);
+    else if (LOG2 > 1 && nsym <= (1 << (LOG2 > 1 ? LOG2 - 1 : 0))) decode_lane<BS, LOG2, OUT, 1, false>(a, s, lp, id.n, rmp);
+    else decode_lane<BS, LOG2, OUT, 0, false>(a, s, lp, id.n, rmp);
+}
+
+}  // namespace

@@ -1,0 +1,347 @@
+// Part of the CacheGen KV codec library for MI355X (gfx950); included by cachegen_hip.hip, which
+// is the one translation unit.  Range encoder: bit writer, coder state, encode_streams_kernel.
+//
+// Paths in the comments are relative to LMCache/ in the reference tree:
+//   enc_new.cu = third_party/torchac_cuda/torchac_kernel_enc_new.cu
+//   dec_new.cu = third_party/torchac_cuda/torchac_kernel_dec_new.cu
+//   cal_cdf.cu = third_party/torchac_cuda/cal_cdf.cu
+//   encoder.py = lmcache/storage_backend/serde/cachegen_encoder.py
+//   decoder.py = lmcache/storage_backend/serde/cachegen_decoder.py
+#pragma once
+
+namespace {
+
+// ---- encoder (enc_new.cu:21-97, 253-307) -------------------------------------------
+// Bits are collected MSB-first in a 64-bit accumulator and leave as big-endian 32-bit words.
+// Every lane of a wavefront runs the store code whenever one lane has a word ready, so words
+// are written at fixed points, once per two symbols, instead of whenever a lane's
+// accumulator fills; the accumulator takes the two symbols in between (a put that would not
+// fit writes a word first).
+// The E1/E2 run of a symbol is emitted at once: the n1 = clz(low ^ high) leading bits
+// agree, and the pending complements go in after the first of them, which in arithmetic
+// is  bits + ((2^pend - 1) << (n1 - 1))  over n1 + pend bits.  The E3 run k is the number
+// of positions below those where low has ones and high has zeros.  One combined shift by
+// n = n1 + k renormalises low and high; n <= 18 for any table whose symbols all have
+// non-zero width, because the span stays above 2^30 between symbols.
+template <bool ALIGNED>
+struct BitWriter {
+    uint8_t *wptr;          // where the next word goes
+    int wstride;            // bytes from one word of the stream to the next (4: contiguous)
+    int cap;
+    int nbytes;
+    uint64_t acc;           // the low `nacc` bits are waiting to be written; bits above are stale
+    int nacc;
+
+    // the last words of a stream that does not fit its slot: keep what fits
+    __device__ __forceinline__ void store_clipped(uint32_t word)
+    {
+        for (int j = 0; j < 4; ++j)
+            if (nbytes + j < cap) wptr[j] = (uint8_t)(word >> (24 - 8 * j));
+    }
+
+    __device__ __forceinline__ void store_word(uint32_t word)
+    {
+        if (__builtin_expect(nbytes + 4 <= cap, 1)) {
+            if (ALIGNED) {
+                *reinterpret_cast<uint32_t *>(wptr) = __builtin_bswap32(word);
+            } else {
+                wptr[0] = (uint8_t)(word >> 24);
+                wptr[1] = (uint8_t)(word >> 16);
+                wptr[2] = (uint8_t)(word >> 8);
+                wptr[3] = (uint8_t)word;
+            }
+        } else {
+            store_clipped(word);
+        }
+        wptr += wstride;
+        nbytes += 4;
+    }
+
+    // write one word if 32 bits are waiting
+    __device__ __forceinline__ void flush_word()
+    {
+        if (nacc >= 32) {
+            store_word((uint32_t)(acc >> (nacc - 32)));
+            nacc -= 32;
+        }
+    }
+
+    // append the low m bits of v (v < 2^m), 0 <= m <= 32 (m = 0 needs v = 0)
+    __device__ __forceinline__ void put(uint32_t v, int m)
+    {
+        if (__builtin_expect(nacc + m > 64, 0)) flush_word();       // more than 32 are waiting then
+        acc = (acc << m) | v;
+        nacc += m;
+    }
+
+    // one bit, then `count` copies of its complement (any count): the general form of
+    // append_bit_and_pending (enc_new.cu:86-97); not on the common path
+    __device__ __forceinline__ void bit_and_run(uint32_t bit, uint32_t count)
+    {
+        uint32_t pv = bit;
+        int pm = 1;
+        for (;;) {
+            put(pv, pm);
+            flush_word();
+            if (count == 0) break;
+            pm = count < 32u ? (int)count : 32;
+            pv = bit ? 0u : (pm == 32 ? 0xFFFFFFFFu : ((1u << pm) - 1u));
+            count -= (uint32_t)pm;
+        }
+    }
+
+    // write what is left, the last partial word byte by byte (enc_new.cu:42-55); returns
+    // the stream length
+    __device__ __forceinline__ int finish()
+    {
+        flush_word();
+        flush_word();
+        if (nacc > 0) {
+            uint32_t r = (uint32_t)(acc << (32 - nacc));
+            for (int left = nacc, j = 0; left > 0; left -= 8, ++j) {
+                if (nbytes < cap) wptr[j] = (uint8_t)(r >> 24);
+                nbytes++;
+                r <<= 8;
+            }
+        }
+        return nbytes;
+    }
+};
+
+// The coder state is (low, span) with span = high - low + 1 held modulo 2^32: 0 stands for
+// the full range 2^32 (the initial state, and any later interval that is exactly a binary
+// fraction), where floor(span * c / 2^16) is simply c << 16.  Renormalising by n bits maps
+// span to span << n for E1/E2 and E3 steps alike.
+template <int BS, bool ALIGNED>
+struct RangeEncoder {
+    const uint16_t *col;    // this lane's table column: entry e at col[e * BS]
+    uint32_t smax;          // lp - 2: the largest symbol
+    uint32_t low, span, pend;
+    BitWriter<ALIGNED> w;
+
+    __device__ __forceinline__ void init(const uint16_t *column, int lp, uint8_t *dst, int wstride, int cap)
+    {
+        col = column;
+        smax = (uint32_t)(lp - 2);
+        low = 0;
+        span = 0;
+        pend = 0;
+        w.wptr = dst;
+        w.wstride = wstride;
+        w.cap = cap;
+        w.nbytes = 0;
+        w.acc = 0;
+        w.nacc = 0;
+    }
+
+    // SENTINEL: symbol smax may occur, whose upper bound is 2^16 and not the table's last
+    // entry (enc_new.cu:270)
+    template <bool SENTINEL>
+    __device__ __forceinline__ void put_symbol(uint32_t s)
+    {
+        s = s < smax ? s : smax;                        // keep table reads inside the table
+        const uint32_t c_lo = col[s * BS];
+        const uint32_t c_next = col[s * BS + BS];
+        const uint32_t c_hi = (SENTINEL && s == smax) ? 0x10000u : c_next;
+        uint32_t t_lo, width;
+        if (__builtin_expect(span == 0, 0)) {
+            t_lo = c_lo << 16;
+            width = (c_hi - c_lo) << 16;
+        } else {
+            const uint32_t sh = span >> 16, sl = span & 0xFFFFu;
+            t_lo = scale_span(sh, sl, c_lo);
+            width = scale_span(sh, sl, c_hi) - t_lo;
+        }
+        low += t_lo;
+        const uint32_t high = low + width - 1u;
+
+        const int n1 = __builtin_clz(low ^ high);       // low < high always
+        // the n1 agreed bits (none if n1 = 0) with the pending complements after the first
+        const uint32_t pe = n1 > 0 ? pend : 0u;
+        const int m = n1 + (int)pe;
+        if (__builtin_expect(m > 32, 0)) {
+            const uint32_t bits = low >> ((32 - n1) & 31);
+            w.bit_and_run(bits >> (n1 - 1), pe);
+            w.put(bits & ((1u << (n1 - 1)) - 1u), n1 - 1);
+        } else {
+            const uint32_t bits = __builtin_amdgcn_ubfe(low, (uint32_t)(32 - n1), (uint32_t)n1);
+            const uint32_t fill = ((1u << (pe & 31)) - 1u) << ((n1 - 1) & 31);
+            w.put(bits + fill, m);
+        }
+        // E3 run: leading zeros of (~low | high) below the first differing bit
+        const uint32_t z = ((low & high) | ~low) << ((n1 + 1) & 31);
+        const int k = __builtin_clz(z);
+        const int n = n1 + k;
+        pend = pend - pe + (uint32_t)k;
+        low = (low << n) & 0x7FFFFFFFu;
+        span = width << n;
+    }
+
+    __device__ __forceinline__ int finish()
+    {
+        pend += 1;
+        w.bit_and_run(low < 0x40000000u ? 0u : 1u, pend);
+        return w.finish();
+    }
+};
+
+struct EncodeArgs {
+    uint16_t *cdf;          // [chunk][row][channel][lp]; written when the histogram is fused
+    int32_t lp;
+    const uint8_t *sym;     // byte symbols: sym[row*s0 + token*s1 + channel*s2]
+    int64_t s0, s1, s2;
+    const uint32_t *sym4;   // or packed symbols
+    int64_t nsub;
+    uint8_t *out;           // out[row*o0 + channel*o1 + byte], or the scratch tiles (SLOTS)
+    int64_t o0, o1;
+    int32_t cap;
+    int32_t *lengths;       // [sub][row][channel]
+    int32_t *status;        // may be null
+    int64_t *tile_sums;     // SLOTS, one block per tile of kSlotTile streams: stored bytes per tile, or null
+    const float *key_bins, *value_bins;     // float32 [L] each, or null when the levels are not known
+    int64_t L;
+    StreamGrid sg;
+};
+
+constexpr int kSlotTile = 256;      // streams per tile of the encoder's scratch
+
+template <bool B>
+struct BoolTag {
+    static constexpr bool value = B;
+};
+
+// PACKED: symbols come from sym4.  FUSE_CDF (PACKED only, one sub-chunk per chunk): the
+// block first builds its own tables from the same words and writes them out.
+// SLOTS: stream g of the launch is written to out[g * cap ...] (the fused path's scratch).
+template <int BS, bool ALIGNED, bool PACKED, bool FUSE_CDF, bool SLOTS>
+__global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
+{
+    extern __shared__ uint16_t tab[];
+    const int tid = threadIdx.x;
+    const StreamId id = locate<BS>(a.sg);
+    const int lp = a.lp;
+    const int64_t ch0 = id.ch - tid;
+    uint16_t *col = tab + tid;
+    uint16_t *cdf_block = a.cdf + ((id.chunk * a.sg.rows + id.row) * a.sg.nc + ch0) * lp;
+    const uint32_t *wp = nullptr;
+    const int nwords = (id.n + 3) >> 2;
+    if (PACKED) wp = a.sym4 + ((id.row * a.nsub + id.sub) * kWordsPerSub) * a.sg.nc + id.ch;
+
+    // PACKED: half a sub-chunk (32 words = 128 symbols) at a time is loaded into registers
+    // and indexed by the (uniform) loop counter, so the coding loop has no loads to wait
+    // for and its stores never hold it up.
+    typedef uint32_t words32 __attribute__((ext_vector_type(32)));
+    words32 words;
+    auto load_half = [&](int h) {
+#pragma unroll
+        for (int w = 0; w < 32; ++w)
+            words[w] = (id.active && h * 32 + w < nwords) ? wp[(int64_t)(h * 32 + w) * a.sg.nc] : 0u;
+    };
+
+    if (FUSE_CDF) {
+        for (int i = 0; i < lp; ++i) col[i * BS] = 0;
+        if (id.active) {
+            const uint32_t smax = (uint32_t)(lp - 2);
+            for (int h = 0; h * 32 < nwords; ++h) {
+                load_half(h);
+                const int wn = nwords - h * 32 < 32 ? nwords - h * 32 : 32;
+#pragma unroll 1
+                for (int w = 0; w < wn; ++w) {
+                    const uint32_t v = words[w];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        uint32_t s = (v >> (8 * j)) & 0xFFu;
+                        s = s < smax ? s : smax;
+                        if ((h * 32 + w) * 4 + j < id.n) col[(s + 1) * BS]++;   // the column is this lane's own
+                    }
+                }
+            }
+            normalize_column16<BS>(col, lp, lp - 1, (uint32_t)id.n);
+        }
+        __syncthreads();
+        write_tables16<BS>(tab, cdf_block, lp, ch0, a.sg.nc);
+    } else {
+        stage_tables16<BS>(tab, cdf_block, lp, ch0, a.sg.nc);
+        __syncthreads();
+    }
+    if (!id.active) return;
+
+    RangeEncoder<BS, ALIGNED> enc;
+    const int64_t stream = (id.sub * a.sg.rows + id.row) * a.sg.nc + id.ch;
+    // SLOTS: the scratch is cut into tiles of kSlotTile streams; word w of a tile's stream t is
+    // the tile's word w * kSlotTile + t, so that the words the lanes of a wavefront write, and
+    // the words the compaction reads, lie side by side
+    if (SLOTS)
+        enc.init(col, lp, a.out + (stream / kSlotTile) * ((int64_t)kSlotTile * a.cap) + (stream % kSlotTile) * 4,
+                 kSlotTile * 4, a.cap);
+    else
+        enc.init(col, lp, a.out + id.row * a.o0 + id.ch * a.o1, 4, a.cap);
+
+    // The row's alphabet (2C + 1 symbols for `bins` levels, encoder.py:44-52) may leave the
+    // table's last symbol unused; then its special upper bound is never needed.  Uniform
+    // over the block.
+    bool sentinel = true;
+    if (PACKED && a.key_bins) {
+        const int64_t kvi = id.row / a.L, l = id.row - kvi * a.L;
+        const float cq = floorf((kvi ? a.value_bins : a.key_bins)[l] * 0.5f) - 1.0f;
+        sentinel = !(cq >= 0.0f && 2.0f * cq + 1.0f <= (float)(lp - 2));
+    }
+
+    auto code = [&](auto tag) {
+        constexpr bool SENTINEL = decltype(tag)::value;
+        if (PACKED) {
+            for (int h = 0; h * 32 < nwords; ++h) {
+                load_half(h);
+                const int wn = nwords - h * 32 < 32 ? nwords - h * 32 : 32;
+#pragma unroll 1
+                for (int w = 0; w < wn; ++w) {
+                    const uint32_t v = words[w];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        if ((h * 32 + w) * 4 + j < id.n) enc.template put_symbol<SENTINEL>((v >> (8 * j)) & 0xFFu);
+                        if (j & 1) enc.w.flush_word();
+                    }
+                }
+            }
+        } else {
+            const uint8_t *sp = a.sym + id.row * a.s0 + id.t0 * a.s1 + id.ch * a.s2;
+            uint32_t nxt[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) nxt[j] = (j < id.n) ? sp[(int64_t)j * a.s1] : 0u;
+            for (int i0 = 0; i0 < id.n; i0 += 8) {
+                uint32_t cur[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) cur[j] = nxt[j];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) nxt[j] = (i0 + 8 + j < id.n) ? sp[(int64_t)(i0 + 8 + j) * a.s1] : 0u;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    if (i0 + j < id.n) enc.template put_symbol<SENTINEL>(cur[j]);
+                    if (j & 1) enc.w.flush_word();
+                }
+            }
+        }
+    };
+    if (PACKED && !sentinel) code(BoolTag<false>());
+    else code(BoolTag<true>());
+    const int len = enc.finish();
+    a.lengths[stream] = len;
+    if (len > a.cap && a.status) atomicOr(a.status, 1);
+    if (SLOTS && a.tile_sums) {
+        // every lane of the block is active here (the host asks for tile sums only when a block
+        // is exactly one tile): bytes the block's streams occupy in the payload
+        __shared__ int32_t wave_sums[BS / 64];
+        int32_t v = len < a.cap ? len : a.cap;
+#pragma unroll
+        for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
+        if ((tid & 63) == 0) wave_sums[tid >> 6] = v;
+        __syncthreads();
+        if (tid == 0) {
+            int64_t total = 0;
+            for (int w = 0; w < BS / 64; ++w) total += wave_sums[w];
+            a.tile_sums[blockIdx.x] = total;
+        }
+    }
+}
+
+}  // namespace

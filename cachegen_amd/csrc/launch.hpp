@@ -1,0 +1,225 @@
+// Part of the CacheGen KV codec library for MI355X (gfx950); included by cachegen_hip.hip, which
+// is the one translation unit.  Host-side launch helpers: block size, grids, kernel dispatch.
+//
+// Paths in the comments are relative to LMCache/ in the reference tree:
+//   enc_new.cu = third_party/torchac_cuda/torchac_kernel_enc_new.cu
+//   dec_new.cu = third_party/torchac_cuda/torchac_kernel_dec_new.cu
+//   cal_cdf.cu = third_party/torchac_cuda/cal_cdf.cu
+//   encoder.py = lmcache/storage_backend/serde/cachegen_encoder.py
+//   decoder.py = lmcache/storage_backend/serde/cachegen_decoder.py
+#pragma once
+
+namespace {
+
+// ------------------------------------------------------------------------------------
+// host-side launch helpers
+// ------------------------------------------------------------------------------------
+// Lanes per block: as many adjacent channels as possible while the per-block table
+// (lp words per lane) stays well inside the default dynamic LDS window.
+int pick_block(int64_t nc, int lp)
+{
+    int block = 256;
+    if (lp > 80) block = 128;
+    while (block > 64 && nc <= block / 2) block /= 2;
+    return block;
+}
+
+int make_grid(int64_t rows, int64_t nc, int64_t T, int64_t S, int64_t nsub, int block,
+              StreamGrid &sg, int64_t &nblocks)
+{
+    sg.rows = rows;
+    sg.nc = nc;
+    sg.ctiles = (int32_t)ceil_div(nc, block);
+    sg.g.T = T;
+    sg.g.S = S;
+    sg.g.nsc = (int32_t)ceil_div(S, kSub);
+    nblocks = nsub * rows * sg.ctiles;
+    if (nblocks <= 0 || nblocks > INT_MAX) return fail(CG_ERR_ARG, "grid of %lld blocks is out of range", (long long)nblocks);
+    return CG_OK;
+}
+
+// Run `launch` with the block size as a compile-time constant.
+#define CG_DISPATCH_BS(block, ...)                      \
+    do {                                                \
+        if ((block) == 256) { constexpr int BS = 256; __VA_ARGS__; } \
+        else if ((block) == 128) { constexpr int BS = 128; __VA_ARGS__; } \
+        else { constexpr int BS = 64; __VA_ARGS__; }    \
+    } while (0)
+
+int launch_cdf(const uint8_t *sym, const uint32_t *sym4, int64_t nsub, int64_t rows, int64_t T,
+               int64_t nc, int64_t s0, int64_t s1, int64_t s2, int max_bins, int64_t S,
+               uint16_t *cdf, hipStream_t stream)
+{
+    const int block = pick_block(nc, max_bins + 1);
+    CdfArgs a;
+    a.sym = sym;
+    a.s0 = s0;
+    a.s1 = s1;
+    a.s2 = s2;
+    a.sym4 = sym4;
+    a.nsub = nsub;
+    a.cdf = cdf;
+    a.rows = rows;
+    a.nc = nc;
+    a.ctiles = (int32_t)ceil_div(nc, block);
+    a.max_bins = max_bins;
+    a.g.T = T;
+    a.g.S = S;
+    a.g.nsc = (int32_t)ceil_div(S, kSub);
+    const int64_t nblocks = ceil_div(T, S) * rows * a.ctiles;
+    if (nblocks <= 0 || nblocks > INT_MAX) return fail(CG_ERR_ARG, "calculate_cdf: grid out of range");
+    const size_t shmem = (size_t)(max_bins + 1) * block * sizeof(uint32_t);
+    const dim3 grid((unsigned)nblocks), blk(block);
+    if (sym4) CG_DISPATCH_BS(block, (calculate_cdf_kernel<BS, true><<<grid, blk, shmem, stream>>>(a)));
+    else CG_DISPATCH_BS(block, (calculate_cdf_kernel<BS, false><<<grid, blk, shmem, stream>>>(a)));
+    return check_launch("calculate_cdf");
+}
+
+int launch_scan(const int32_t *lengths, int64_t n, int32_t clamp, int64_t *offsets, void *scratch,
+                hipStream_t stream)
+{
+    const int64_t ntiles = ceil_div(n, kScanTile);
+    int64_t *sums = static_cast<int64_t *>(scratch);
+    scan_tile_sums_kernel<<<dim3((unsigned)ntiles), dim3(kScanThreads), 0, stream>>>(lengths, n, clamp, sums);
+    scan_sums_kernel<<<dim3(1), dim3(kScanThreads), 0, stream>>>(sums, ntiles);
+    scan_apply_kernel<<<dim3((unsigned)ntiles), dim3(kScanThreads), 0, stream>>>(lengths, n, clamp, sums, offsets);
+    return check_launch("scan_lengths");
+}
+
+int check_dt(int dt, const char *what)
+{
+    if (dt != CG_DT_F16 && dt != CG_DT_BF16) return fail(CG_ERR_ARG, "%s: dtype must be CG_DT_F16 or CG_DT_BF16", what);
+    return CG_OK;
+}
+
+int check_lp(int lp, const char *what)
+{
+    if (lp < 2 || lp > CG_MAX_LP) return fail(CG_ERR_ARG, "%s: CDF length should be in [2, %d], got %d", what, CG_MAX_LP, lp);
+    return CG_OK;
+}
+
+bool kv_vectorizable(const void *kv, int64_t D, int64_t C, int64_t sl, int64_t skv, int64_t st, int64_t sh)
+{
+    return (D % 8 == 0) && (sl % 8 == 0) && (skv % 8 == 0) && (st % 8 == 0) && (sh % 8 == 0) &&
+           aligned_to(kv, 16) && (C / 8 <= 64 * kMaxUnits);
+}
+
+int launch_quantize(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D,
+                    int64_t sl, int64_t skv, int64_t st, int64_t sh, const float *key_bins,
+                    const float *value_bins, uint8_t *sym, void *maxima, hipStream_t stream)
+{
+    const int64_t C = H * D;
+    const int64_t nrows = 2 * L * T;
+    const int64_t nblocks = ceil_div(nrows, 4);
+    if (nblocks > INT_MAX || C > INT_MAX) return fail(CG_ERR_ARG, "quantize: tensor too large for one launch");
+    const bool vec = kv_vectorizable(kv, D, C, sl, skv, st, sh) && aligned_to(sym, 8);
+    const uint16_t *p = static_cast<const uint16_t *>(kv);
+    uint16_t *mx = static_cast<uint16_t *>(maxima);
+    dim3 grid((unsigned)nblocks), block(256);
+    if (vec) {
+        const int nunits = (int)(C / 8);
+        const bool contiguous = (sh == D);
+#define CG_LAUNCH_Q(DT, HC) quantize_kv_kernel<DT, HC><<<grid, block, 0, stream>>>( \
+        p, L, T, (int)D, sl, skv, st, sh, key_bins, value_bins, sym, mx, nunits, nrows)
+        if (kv_dt == CG_DT_F16) { if (contiguous) CG_LAUNCH_Q(CG_DT_F16, true); else CG_LAUNCH_Q(CG_DT_F16, false); }
+        else { if (contiguous) CG_LAUNCH_Q(CG_DT_BF16, true); else CG_LAUNCH_Q(CG_DT_BF16, false); }
+#undef CG_LAUNCH_Q
+    } else {
+        if (kv_dt == CG_DT_F16)
+            quantize_kv_generic_kernel<CG_DT_F16><<<grid, block, 0, stream>>>(
+                p, L, T, (int)D, (int)C, sl, skv, st, sh, key_bins, value_bins, sym, mx, nrows);
+        else
+            quantize_kv_generic_kernel<CG_DT_BF16><<<grid, block, 0, stream>>>(
+                p, L, T, (int)D, (int)C, sl, skv, st, sh, key_bins, value_bins, sym, mx, nrows);
+    }
+    return check_launch("quantize_kv");
+}
+
+template <int DT, bool HC>
+void launch_quantize_pack_nu(const PackedQuantArgs &a, int64_t nblocks, hipStream_t stream)
+{
+    const dim3 grid((unsigned)nblocks), block(256);
+    if (a.delta_group > 0) {
+        if (a.nunits <= 128) quantize_pack_delta_kernel<DT, HC, 2><<<grid, block, 0, stream>>>(a);
+        else if (a.nunits <= 256) quantize_pack_delta_kernel<DT, HC, 4><<<grid, block, 0, stream>>>(a);
+        else quantize_pack_delta_kernel<DT, HC, 8><<<grid, block, 0, stream>>>(a);
+        return;
+    }
+    if (a.nunits <= 128) quantize_pack_kernel<DT, HC, 2><<<grid, block, 0, stream>>>(a);
+    else if (a.nunits <= 256) quantize_pack_kernel<DT, HC, 4><<<grid, block, 0, stream>>>(a);
+    else quantize_pack_kernel<DT, HC, 8><<<grid, block, 0, stream>>>(a);
+}
+
+int launch_quantize_pack(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D,
+                         int64_t sl, int64_t skv, int64_t st, int64_t sh, const float *key_bins,
+                         const float *value_bins, uint32_t *sym4, void *maxima, int64_t nsub,
+                         int64_t S, int delta_group, hipStream_t stream)
+{
+    PackedQuantArgs a;
+    a.kv = static_cast<const uint16_t *>(kv);
+    a.L = L;
+    a.sl = sl;
+    a.skv = skv;
+    a.st = st;
+    a.sh = sh;
+    a.D = (int32_t)D;
+    a.key_bins = key_bins;
+    a.value_bins = value_bins;
+    a.sym4 = sym4;
+    a.maxima = static_cast<uint16_t *>(maxima);
+    a.nunits = (int32_t)(H * D / 8);
+    a.nsub = nsub;
+    a.delta_group = delta_group;
+    a.g.T = T;
+    a.g.S = S;
+    a.g.nsc = (int32_t)ceil_div(S, kSub);
+    const int64_t nblocks = 2 * L * nsub * 16;
+    if (nblocks > INT_MAX) return fail(CG_ERR_ARG, "quantize: tensor too large for one launch");
+    const bool contiguous = (sh == D);
+    if (kv_dt == CG_DT_F16) {
+        if (contiguous) launch_quantize_pack_nu<CG_DT_F16, true>(a, nblocks, stream);
+        else launch_quantize_pack_nu<CG_DT_F16, false>(a, nblocks, stream);
+    } else {
+        if (contiguous) launch_quantize_pack_nu<CG_DT_BF16, true>(a, nblocks, stream);
+        else launch_quantize_pack_nu<CG_DT_BF16, false>(a, nblocks, stream);
+    }
+    return check_launch("quantize_pack");
+}
+
+// Describe the readable byte window [bytes, bytes + nbytes) to the bit reader, which
+// loads aligned words at 32-bit offsets from the window's 4-byte-aligned base.
+int set_byte_window(DecodeArgs &a, const uint8_t *bytes, int64_t nbytes, const char *what)
+{
+    if (nbytes <= 0) return fail(CG_ERR_ARG, "%s: empty byte buffer", what);
+    const uint32_t skew = (uint32_t)(reinterpret_cast<uintptr_t>(bytes) & 3u);
+    a.bytes = bytes - skew;
+    a.bytes_skew = skew;
+    a.last_word = (skew + nbytes - 1) & ~3ll;
+    return CG_OK;
+}
+
+size_t decode_shmem(int lp, int block) { return align_up((size_t)lp * block * sizeof(uint16_t), 4) + (size_t)(lp + kSub) * sizeof(float); }
+
+template <int SRC>
+int launch_decode_symbols(const DecodeArgs &a, int64_t nblocks, int block, hipStream_t stream)
+{
+    const dim3 grid((unsigned)nblocks), blk(block);
+    const size_t shmem = decode_shmem(a.lp, block);
+    CG_DISPATCH_BS(block, (decode_streams_kernel<BS, -1, SRC, OUT_SYMBOLS><<<grid, blk, shmem, stream>>>(a)));
+    return check_launch("decode");
+}
+
+template <int BS, int OUT>
+void launch_decode_kv_log2(const DecodeArgs &a, dim3 grid, size_t shmem, hipStream_t stream)
+{
+    const dim3 blk(BS);
+    switch (a.lp) {
+    case 9: decode_streams_kernel<BS, 3, SRC_OFFSETS, OUT><<<grid, blk, shmem, stream>>>(a); break;
+    case 17: decode_streams_kernel<BS, 4, SRC_OFFSETS, OUT><<<grid, blk, shmem, stream>>>(a); break;
+    case 33: decode_streams_kernel<BS, 5, SRC_OFFSETS, OUT><<<grid, blk, shmem, stream>>>(a); break;
+    case 65: decode_streams_kernel<BS, 6, SRC_OFFSETS, OUT><<<grid, blk, shmem, stream>>>(a); break;
+    default: decode_streams_kernel<BS, -1, SRC_OFFSETS, OUT><<<grid, blk, shmem, stream>>>(a); break;
+    }
+}
+
+}  // namespace

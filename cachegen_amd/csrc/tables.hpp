@@ -1,0 +1,221 @@
+// Part of the CacheGen KV codec library for MI355X (gfx950); included by cachegen_hip.hip, which
+// is the one translation unit.  Per-(row, channel) tables: histogram, running sum, normalisation, staging in LDS; block-to-stream geometry.
+//
+// Paths in the comments are relative to LMCache/ in the reference tree:
+//   enc_new.cu = third_party/torchac_cuda/torchac_kernel_enc_new.cu
+//   dec_new.cu = third_party/torchac_cuda/torchac_kernel_dec_new.cu
+//   cal_cdf.cu = third_party/torchac_cuda/cal_cdf.cu
+//   encoder.py = lmcache/storage_backend/serde/cachegen_encoder.py
+//   decoder.py = lmcache/storage_backend/serde/cachegen_decoder.py
+#pragma once
+
+namespace {
+
+// ------------------------------------------------------------------------------------
+// Tables (cal_cdf.cu:17-59): one lane per (chunk, row, channel) walks the chunk's tokens
+// and counts into its own LDS column hist[bin][lane] (no atomics across lanes, no bank
+// conflicts); the running sum and the normalisation
+//   cdf[i] = (uint16)((0xFFFF - max_bins) * cum[i] / cum[max_bins]) + i
+// are done per lane in 16-bit wrap-around arithmetic like the reference's uint16
+// counters, and the block writes its tables back transposed so stores coalesce.
+// ------------------------------------------------------------------------------------
+
+// Running sum and normalisation of one lane's column col[i * BS], i in [0, lp).
+template <int BS>
+__device__ __forceinline__ void normalize_column(uint32_t *col, int lp, int max_bins)
+{
+    uint32_t running = 0;
+    for (int i = 1; i < lp; ++i) {
+        running = (running + col[i * BS]) & 0xFFFFu;
+        col[i * BS] = running;
+    }
+    const uint32_t scale = 0xFFFFu - (uint32_t)max_bins;
+    for (int i = 0; i < lp; ++i) {
+        const uint32_t q = running ? (scale * col[i * BS] / running) & 0xFFFFu : 0u;
+        col[i * BS] = (q + (uint32_t)i) & 0xFFFFu;
+    }
+}
+
+// Write the block's tables tab[entry * BS + lane] to cdf[lane][entry], coalesced.
+template <int BS>
+__device__ __forceinline__ void write_tables(const uint32_t *tab, uint16_t *cdf, int lp, int64_t ch0, int64_t nc)
+{
+    const int64_t nvalid = (nc - ch0 < BS) ? (nc - ch0) : BS;
+    const int total = (int)nvalid * lp;
+    for (int i = threadIdx.x; i < total; i += BS) {
+        const int c = i / lp, e = i - c * lp;
+        cdf[i] = (uint16_t)tab[e * BS + c];
+    }
+}
+
+// Load the block's tables into LDS as tab[entry * BS + lane] (32-bit words).
+template <int BS>
+__device__ __forceinline__ void stage_tables(uint32_t *tab, const uint16_t *cdf, int lp, int64_t ch0, int64_t nc)
+{
+    const int64_t nvalid = (nc - ch0 < BS) ? (nc - ch0) : BS;
+    const int total = (int)nvalid * lp;
+    for (int i = threadIdx.x; i < total; i += BS) {
+        const int c = i / lp, e = i - c * lp;
+        tab[e * BS + c] = cdf[i];
+    }
+}
+
+// The stream kernels keep their tables in LDS as 16-bit entries tab[entry * BS + lane]
+// (half the footprint, twice the resident waves).  The end of a table, 2^16, does not fit
+// and is substituted where the last symbol's upper bound is read.
+template <int BS>
+__device__ __forceinline__ void stage_tables16(uint16_t *tab, const uint16_t *cdf, int lp, int64_t ch0, int64_t nc)
+{
+    const int64_t nvalid = (nc - ch0 < BS) ? (nc - ch0) : BS;
+    const int total = (int)nvalid * lp;
+    for (int i = threadIdx.x; i < total; i += BS) {
+        const int c = i / lp, e = i - c * lp;
+        tab[e * BS + c] = cdf[i];
+    }
+}
+
+template <int BS>
+__device__ __forceinline__ void write_tables16(const uint16_t *tab, uint16_t *cdf, int lp, int64_t ch0, int64_t nc)
+{
+    const int64_t nvalid = (nc - ch0 < BS) ? (nc - ch0) : BS;
+    const int total = (int)nvalid * lp;
+    for (int i = threadIdx.x; i < total; i += BS) {
+        const int c = i / lp, e = i - c * lp;
+        cdf[i] = tab[e * BS + c];
+    }
+}
+
+// Running sum and normalisation of one lane's 16-bit column of counts when every one of
+// `total` tokens was counted (1 <= total <= 65535, uniform over the block): the divide of
+// cal_cdf.cu:11-14 becomes a shift or a float estimate corrected exactly.
+template <int BS>
+__device__ __forceinline__ void normalize_column16(uint16_t *col, int lp, int max_bins, uint32_t total)
+{
+    const uint32_t scale = 0xFFFFu - (uint32_t)max_bins;
+    uint32_t running = 0;
+    if ((total & (total - 1)) == 0) {
+        const int sh = 31 - __builtin_clz(total);
+        for (int i = 0; i < lp; ++i) {
+            running += col[i * BS];
+            col[i * BS] = (uint16_t)(((scale * running) >> sh) + (uint32_t)i);
+        }
+    } else {
+        const float inv = __fdiv_rn(1.0f, (float)total);
+        for (int i = 0; i < lp; ++i) {
+            running += col[i * BS];
+            const uint32_t x = scale * running;                  // < 2^32, quotient < 2^16
+            uint32_t q = (uint32_t)((float)x * inv);
+            int32_t rem = (int32_t)(x - q * total);
+            if (rem < 0) { q--; rem += (int32_t)total; }
+            if (rem >= (int32_t)total) q++;
+            col[i * BS] = (uint16_t)(q + (uint32_t)i);
+        }
+    }
+}
+
+struct CdfArgs {
+    const uint8_t *sym;     // byte symbols: sym[row*s0 + token*s1 + channel*s2]
+    int64_t s0, s1, s2;
+    const uint32_t *sym4;   // or packed symbols (see above)
+    int64_t nsub;
+    uint16_t *cdf;          // [chunk][row][channel][lp]
+    int64_t rows, nc;
+    int32_t ctiles;
+    int32_t max_bins;
+    TokenGeom g;
+};
+
+template <int BS, bool PACKED>
+__global__ __launch_bounds__(BS) void calculate_cdf_kernel(CdfArgs a)
+{
+    extern __shared__ uint32_t smem[];
+    const int tid = threadIdx.x;
+    const int lp = a.max_bins + 1;
+    int64_t b = blockIdx.x;
+    const int ctile = (int)(b % a.ctiles);
+    b /= a.ctiles;
+    const int64_t row = b % a.rows;
+    const int64_t chunk = b / a.rows;
+    const int64_t ch = (int64_t)ctile * BS + tid;
+    uint32_t *col = smem + tid;
+    for (int i = 0; i < lp; ++i) col[i * BS] = 0;
+
+    const int64_t t0 = chunk * a.g.S;
+    int64_t t1 = t0 + a.g.S;
+    if (t1 > a.g.T) t1 = a.g.T;
+    const uint32_t mb = (uint32_t)a.max_bins;
+    if (ch < a.nc) {
+        if (!PACKED) {
+            const uint8_t *p = a.sym + row * a.s0 + ch * a.s2;
+            int64_t t = t0;
+            for (; t + 8 <= t1; t += 8) {
+                uint32_t v[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) v[j] = p[(t + j) * a.s1];
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (v[j] < mb) col[(v[j] + 1) * BS]++;
+            }
+            for (; t < t1; ++t) {
+                const uint32_t v = p[t * a.s1];
+                if (v < mb) col[(v + 1) * BS]++;
+            }
+        } else {
+            const int64_t sub0 = chunk * a.g.nsc;
+            const int nsubs = (int)((t1 - t0 + kSub - 1) / kSub);
+            for (int sidx = 0; sidx < nsubs; ++sidx) {
+                const int64_t left = (t1 - t0) - (int64_t)sidx * kSub;
+                const int n = left < kSub ? (int)left : kSub;
+                const uint32_t *wp = a.sym4 + ((row * a.nsub + sub0 + sidx) * kWordsPerSub) * a.nc + ch;
+                const int nwords = (n + 3) >> 2;
+                for (int w0 = 0; w0 < nwords; w0 += 4) {
+                    uint32_t v[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) v[j] = (w0 + j < nwords) ? wp[(int64_t)(w0 + j) * a.nc] : 0u;
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) {
+                        const uint32_t s = (v[j >> 2] >> (8 * (j & 3))) & 0xFFu;
+                        if (w0 * 4 + j < n && s < mb) col[(s + 1) * BS]++;
+                    }
+                }
+            }
+        }
+        normalize_column<BS>(col, lp, a.max_bins);
+    }
+    __syncthreads();
+    const int64_t ch0 = (int64_t)ctile * BS;
+    write_tables<BS>(smem, a.cdf + ((chunk * a.rows + row) * a.nc + ch0) * lp, lp, ch0, a.nc);
+}
+
+// ------------------------------------------------------------------------------------
+// Arithmetic coder.  Shared geometry of the encoder and decoder kernels: a block of BS
+// lanes covers BS adjacent channels of one (sub-chunk, row).
+// ------------------------------------------------------------------------------------
+struct StreamGrid {
+    int64_t rows, nc;
+    int32_t ctiles;
+    TokenGeom g;
+};
+
+struct StreamId {
+    int64_t sub, row, chunk, t0, ch;
+    int n;
+    bool active;
+};
+
+template <int BS>
+__device__ __forceinline__ StreamId locate(const StreamGrid &sg)
+{
+    StreamId s;
+    int64_t b = blockIdx.x;
+    const int ctile = (int)(b % sg.ctiles);
+    b /= sg.ctiles;
+    s.row = b % sg.rows;
+    s.sub = b / sg.rows;
+    sub_range(sg.g, s.sub, s.chunk, s.t0, s.n);
+    s.ch = (int64_t)ctile * BS + threadIdx.x;
+    s.active = s.ch < sg.nc;
+    return s;
+}
+
+}  // namespace

@@ -42,11 +42,17 @@ def encode_function(kv: torch.Tensor, config: CacheGenConfig, key_bins: torch.Te
     num_heads, head_size = kv.shape[-2:]
     enc = codec.encode_kv(kv, key_bins, value_bins, chunk_tokens=chunk_size, fmt="vllm")
     enc.check()
-    cdf, max_k, max_v, subs = enc.chunk(0)
-    data_chunks = [CacheGenGPUBytestream(bytestream=b, bytestream_lengths=l, ntokens=n)
+    return _chunk_output(enc, 0, enc.sub_boundaries(), num_heads, head_size)
+
+
+def _chunk_output(enc, i, bounds, num_heads, head_size) -> CacheGenGPUEncoderOutput:
+    """Chunk i of an encoded tensor as the reference's container.  Every field is a tensor of
+    its own: pickling a view would write out the whole buffer it is a view of."""
+    cdf, max_k, max_v, subs = enc.chunk(i, bounds)
+    data_chunks = [CacheGenGPUBytestream(bytestream=b.clone(), bytestream_lengths=l.clone(), ntokens=n)
                    for b, l, n in subs]
-    return CacheGenGPUEncoderOutput(data_chunks, cdf, max_tensors_key=max_k, max_tensors_value=max_v,
-                                    num_heads=num_heads, head_size=head_size)
+    return CacheGenGPUEncoderOutput(data_chunks, cdf.clone(), max_tensors_key=max_k.clone(),
+                                    max_tensors_value=max_v.clone(), num_heads=num_heads, head_size=head_size)
 
 
 class CacheGenSerializer(Serializer):
@@ -96,10 +102,4 @@ class CacheGenSerializer(Serializer):
             return wire.pack_chunks(enc)
         enc.check()
         bounds = enc.sub_boundaries()
-        blobs = []
-        for i in range(enc.num_chunks):
-            cdf, max_k, max_v, subs = enc.chunk(i, bounds)
-            data_chunks = [CacheGenGPUBytestream(bytestream=b, bytestream_lengths=l, ntokens=n) for b, l, n in subs]
-            blobs.append(CacheGenGPUEncoderOutput(data_chunks, cdf, max_tensors_key=max_k, max_tensors_value=max_v,
-                                                  num_heads=num_heads, head_size=head_size).to_bytes())
-        return blobs
+        return [_chunk_output(enc, i, bounds, num_heads, head_size).to_bytes() for i in range(enc.num_chunks)]

@@ -147,7 +147,7 @@ def test_flat_serde_decodes_to_the_same_tensor_as_the_pickle_serde(fmt):
             kv = kv.permute(0, 1, 3, 2, 4).contiguous()
         a, b = s_ref.to_bytes(kv), s_flat.to_bytes(kv)
         assert wire.is_flat(b) and not wire.is_flat(a)
-        assert len(b) < len(a) + 512
+        assert len(b) < len(a) + 512 and len(a) < len(b) + 8192     # neither container carries dead bytes
         ta, tb = d.from_bytes(a), d.from_bytes(b)
         assert ta.shape == kv.shape and ta.dtype == tb.dtype
         assert torch.equal(ta.view(torch.int16), tb.view(torch.int16))

@@ -66,10 +66,12 @@ struct BitWriter {
         }
     }
 
-    // append the low m bits of v (v < 2^m), 0 <= m <= 32 (m = 0 needs v = 0)
+    // append the low m bits of v (v < 2^m), 0 <= m <= 32 (m = 0 needs v = 0).  ROOM: the caller
+    // knows that at most 32 bits are waiting (it has just called flush_word), so they fit.
+    template <bool ROOM = false>
     __device__ __forceinline__ void put(uint32_t v, int m)
     {
-        if (__builtin_expect(nacc + m > 64, 0)) flush_word();       // more than 32 are waiting then
+        if (!ROOM && __builtin_expect(nacc + m > 64, 0)) flush_word();   // more than 32 are waiting then
         acc = (acc << m) | v;
         nacc += m;
     }
@@ -136,7 +138,8 @@ struct RangeEncoder {
 
     // SENTINEL: symbol smax may occur, whose upper bound is 2^16 and not the table's last
     // entry (enc_new.cu:270)
-    template <bool SENTINEL>
+    // FIRST: the symbol directly follows a flush_word (the first of a pair)
+    template <bool SENTINEL, bool FIRST>
     __device__ __forceinline__ void put_symbol(uint32_t s)
     {
         s = s < smax ? s : smax;                        // keep table reads inside the table
@@ -166,7 +169,7 @@ struct RangeEncoder {
         } else {
             const uint32_t bits = __builtin_amdgcn_ubfe(low, (uint32_t)(32 - n1), (uint32_t)n1);
             const uint32_t fill = ((1u << (pe & 31)) - 1u) << ((n1 - 1) & 31);
-            w.put(bits + fill, m);
+            w.template put<FIRST>(bits + fill, m);
         }
         // E3 run: leading zeros of (~low | high) below the first differing bit
         const uint32_t z = ((low & high) | ~low) << ((n1 + 1) & 31);
@@ -296,11 +299,13 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
 #pragma unroll 1
                 for (int w = 0; w < wn; ++w) {
                     const uint32_t v = words[w];
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        if ((h * 32 + w) * 4 + j < id.n) enc.template put_symbol<SENTINEL>((v >> (8 * j)) & 0xFFu);
-                        if (j & 1) enc.w.flush_word();
-                    }
+                    const int t = (h * 32 + w) * 4;            // first token of the word
+                    if (t + 0 < id.n) enc.template put_symbol<SENTINEL, true>(v & 0xFFu);
+                    if (t + 1 < id.n) enc.template put_symbol<SENTINEL, false>((v >> 8) & 0xFFu);
+                    enc.w.flush_word();
+                    if (t + 2 < id.n) enc.template put_symbol<SENTINEL, true>((v >> 16) & 0xFFu);
+                    if (t + 3 < id.n) enc.template put_symbol<SENTINEL, false>(v >> 24);
+                    enc.w.flush_word();
                 }
             }
         } else {
@@ -315,9 +320,10 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
 #pragma unroll
                 for (int j = 0; j < 8; ++j) nxt[j] = (i0 + 8 + j < id.n) ? sp[(int64_t)(i0 + 8 + j) * a.s1] : 0u;
 #pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    if (i0 + j < id.n) enc.template put_symbol<SENTINEL>(cur[j]);
-                    if (j & 1) enc.w.flush_word();
+                for (int j = 0; j < 8; j += 2) {
+                    if (i0 + j < id.n) enc.template put_symbol<SENTINEL, true>(cur[j]);
+                    if (i0 + j + 1 < id.n) enc.template put_symbol<SENTINEL, false>(cur[j + 1]);
+                    enc.w.flush_word();
                 }
             }
         }

@@ -82,3 +82,28 @@ def test_bench_refuses_more_than_one_gpu():
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"],
                        capture_output=True, text=True)
     assert r.returncode != 0 and "one GPU" in r.stderr
+
+
+def test_missing_library_is_a_loud_error(monkeypatch, tmp_path):
+    """No fallback: without the built library every entry of the product path raises."""
+    import torch
+    from cachegen_amd import _lib, codec
+    monkeypatch.setattr(_lib, "_handle", None)
+    monkeypatch.setattr(_lib, "LIBRARY", str(tmp_path / "libcachegen_hip.so"))
+    with pytest.raises(RuntimeError, match="is missing"):
+        _lib.lib()
+    with pytest.raises(RuntimeError, match="is missing"):
+        codec.num_subchunks(512, 256)
+    with pytest.raises(RuntimeError, match="should be on GPU"):
+        codec.encode_kv(torch.zeros((1, 2, 4, 1, 8), dtype=torch.float16), torch.ones(1), torch.ones(1))
+
+
+def test_product_code_never_touches_the_oracle():
+    """The oracle is test infrastructure: nothing under cachegen_amd/ names it."""
+    import os
+    root = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "cachegen_amd")
+    for folder, _, files in os.walk(root):
+        for name in files:
+            if name.endswith((".py", ".hip", ".hpp", ".h")):
+                text = open(os.path.join(folder, name)).read()
+                assert "oracle" not in text.replace("no reference to be at parity", ""), os.path.join(folder, name)

@@ -245,6 +245,10 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
         for (int i = 0; i < lp; ++i) col[i * BS] = 0;
         if (id.active) {
             const uint32_t smax = (uint32_t)(lp - 2);
+            // two lanes share a 32-bit LDS word: each adds to its own half with one atomic that
+            // returns nothing (a count is at most 256, so the low half never carries over)
+            uint32_t *const pair = reinterpret_cast<uint32_t *>(tab) + (tid >> 1);
+            const uint32_t one = (tid & 1) ? 0x10000u : 1u;
             for (int h = 0; h * 32 < nwords; ++h) {
                 load_half(h);
                 const int wn = nwords - h * 32 < 32 ? nwords - h * 32 : 32;
@@ -255,7 +259,7 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
                     for (int j = 0; j < 4; ++j) {
                         uint32_t s = (v >> (8 * j)) & 0xFFu;
                         s = s < smax ? s : smax;
-                        if ((h * 32 + w) * 4 + j < id.n) col[(s + 1) * BS]++;   // the column is this lane's own
+                        if ((h * 32 + w) * 4 + j < id.n) atomicAdd(pair + (s + 1) * (BS / 2), one);
                     }
                 }
             }

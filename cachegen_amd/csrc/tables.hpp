@@ -154,11 +154,11 @@ __global__ __launch_bounds__(BS) void calculate_cdf_kernel(CdfArgs a)
                 for (int j = 0; j < 8; ++j) v[j] = p[(t + j) * a.s1];
 #pragma unroll
                 for (int j = 0; j < 8; ++j)
-                    if (v[j] < mb) col[(v[j] + 1) * BS]++;
+                    if (v[j] < mb) atomicAdd(col + (v[j] + 1) * BS, 1u);      // no value returned: one LDS operation
             }
             for (; t < t1; ++t) {
                 const uint32_t v = p[t * a.s1];
-                if (v < mb) col[(v + 1) * BS]++;
+                if (v < mb) atomicAdd(col + (v + 1) * BS, 1u);
             }
         } else {
             const int64_t sub0 = chunk * a.g.nsc;
@@ -175,7 +175,7 @@ __global__ __launch_bounds__(BS) void calculate_cdf_kernel(CdfArgs a)
 #pragma unroll
                     for (int j = 0; j < 16; ++j) {
                         const uint32_t s = (v[j >> 2] >> (8 * (j & 3))) & 0xFFu;
-                        if (w0 * 4 + j < n && s < mb) col[(s + 1) * BS]++;
+                        if (w0 * 4 + j < n && s < mb) atomicAdd(col + (s + 1) * BS, 1u);
                     }
                 }
             }

@@ -74,17 +74,17 @@ def level_bins(level: int, model_name: str = "mistralai/Mistral-7B-Instruct-v0.2
 
 
 def encode_levels(kv: torch.Tensor, chunk_size: int, levels: Sequence[int] = QUANT_LEVELS, fmt: str = "vllm",
-                  model_name: str = "mistralai/Mistral-7B-Instruct-v0.2") -> List[Dict[int, bytes]]:
+                  model_name: str = "mistralai/Mistral-7B-Instruct-v0.2", compact: bool = True) -> List[Dict[int, bytes]]:
     """What the encode half of run_adaptation.py:63-72 leaves on disk, kept in memory:
-    blobs[chunk][level] = the chunk's flat wire container at that level.  The cache is read once
-    per level for all of its chunks."""
+    blobs[chunk][level] = the chunk's flat wire container at that level (version 2 unless
+    compact=False).  The cache is read once per level for all of its chunks."""
     from . import codec
     from .serde import wire
     tables = [level_bins(level, model_name) for level in levels]
     encoded = codec.encode_kv_levels(kv, tables, chunk_tokens=chunk_size, fmt=fmt)
     blobs: List[Dict[int, bytes]] = [dict() for _ in range(encoded[0].num_chunks)]
     for level, enc in zip(levels, encoded):
-        for i, blob in enumerate(wire.pack_chunks(enc)):
+        for i, blob in enumerate(wire.pack_chunks(enc, compact=compact)):
             blobs[i][level] = blob
     return blobs
 

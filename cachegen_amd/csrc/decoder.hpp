@@ -51,7 +51,7 @@ struct BitReader {
     {
         // a start outside the buffer (offsets that are not running sums of stream lengths) is
         // moved inside it: such a stream decodes to garbage, never to a read out of bounds
-        begin = begin < 0 ? 0 : (begin > last_word ? last_word : begin);
+        begin = begin < 0 ? 0 : (begin > last_word + 3 ? last_word + 3 : begin);     // last_word is a word's first byte
         const uint32_t skip = (uint32_t)begin & 3u;
         const int64_t first_word = begin - skip;
         base = window + first_word;

@@ -3,6 +3,7 @@
   "torch"          the chunk tensor as torch.save writes it
   "cachegen"       the codec, in the reference's pickle container
   "cachegen-flat"  the same codec in the flat container of `wire` (not in the reference)
+  "cachegen-compact"  the same in version 2 of that container (tables as histogram counts)
 """
 from ..config import GlobalConfig, LMCacheEngineConfig, LMCacheEngineMetadata
 from .cachegen_decoder import CacheGenDeserializer
@@ -16,6 +17,8 @@ _FACTORIES = {
                                           CacheGenDeserializer(config, metadata)),
     "cachegen-flat": lambda config, metadata: (CacheGenSerializer(config, metadata, wire_format="flat"),
                                                CacheGenDeserializer(config, metadata)),
+    "cachegen-compact": lambda config, metadata: (CacheGenSerializer(config, metadata, wire_format="compact"),
+                                                  CacheGenDeserializer(config, metadata)),
 }
 
 

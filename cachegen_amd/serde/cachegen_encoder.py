@@ -59,9 +59,10 @@ class CacheGenSerializer(Serializer):
     def __init__(self, config: LMCacheEngineConfig, metadata: LMCacheEngineMetadata,
                  wire_format: str = "pickle"):
         """wire_format "pickle": the reference's container (cachegen_basics.py:110-122);
-        "flat": the versioned flat container of `wire`, which `CacheGenDeserializer` reads
-        as well."""
-        if wire_format not in ("pickle", "flat"):
+        "flat": the versioned flat container of `wire`; "compact": its version 2, which stores
+        the tables of chunks of up to 256 tokens as histogram counts.  `CacheGenDeserializer`
+        reads all three."""
+        if wire_format not in ("pickle", "flat", "compact"):
             raise ValueError(f"Invalid wire format: {wire_format}")
         self.wire_format = wire_format
         self.cachegen_config = CacheGenConfig.from_model_name(metadata.model_name)
@@ -83,9 +84,9 @@ class CacheGenSerializer(Serializer):
         if self.fmt == "huggingface":
             tensor = tensor.permute(0, 1, 3, 2, 4)
         ntokens = tensor.shape[2]
-        if self.wire_format == "flat":
+        if self.wire_format != "pickle":
             enc = codec.encode_kv(tensor.cuda(), self.key_bins, self.value_bins, chunk_tokens=ntokens)
-            return wire.pack_chunks(enc, per_chunk=False)[0]
+            return wire.pack_chunks(enc, per_chunk=False, compact=self.wire_format == "compact")[0]
         output = encode_function(tensor.cuda(), self.cachegen_config, self.key_bins,
                                  self.value_bins, ntokens)
         return output.to_bytes()
@@ -98,8 +99,8 @@ class CacheGenSerializer(Serializer):
             tensor = tensor.permute(0, 1, 3, 2, 4)
         num_heads, head_size = tensor.shape[-2:]
         enc = codec.encode_kv(tensor.cuda(), self.key_bins, self.value_bins, chunk_tokens=chunk_size)
-        if self.wire_format == "flat":
-            return wire.pack_chunks(enc)
+        if self.wire_format != "pickle":
+            return wire.pack_chunks(enc, compact=self.wire_format == "compact")
         enc.check()
         bounds = enc.sub_boundaries()
         return [_chunk_output(enc, i, bounds, num_heads, head_size).to_bytes() for i in range(enc.num_chunks)]

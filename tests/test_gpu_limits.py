@@ -167,3 +167,26 @@ def test_nan_and_infinite_rows_match_oracle(oracle):
             nan_got, nan_ref = (got & 0x7FFF) > inf_bits, (ref & 0x7FFF) > inf_bits
             assert np.array_equal(nan_got, nan_ref), (dtype, out_dtype)
             assert nan_ref.any() and np.array_equal(got[~nan_ref], ref[~nan_ref]), (dtype, out_dtype)
+
+
+@pytest.mark.parametrize("nt", [1, 2, 7])
+def test_streams_that_begin_in_the_last_word_of_an_exact_size_buffer(oracle, nt):
+    """The byte buffer ends with the last stream, and that stream is so short that it starts
+    inside the buffer's last 32-bit word."""
+    _, tac = _mods()
+    rng = np.random.default_rng(nt)
+    nl, nc = 3, 5
+    sym = rng.integers(0, 3, size=(nl, nt, nc), dtype=np.uint8)           # cheap symbols: 1-2 byte streams
+    table = np.tile(rng.integers(0, 3, size=(nl, 300, nc), dtype=np.uint8), (1, 1, 1))
+    cdf = oracle.calculate_cdf(table, 32)
+    pad, lens = oracle.encode_fast_new(cdf, sym)
+    data = oracle.collect_bytes(pad, lens)
+    assert lens.max() <= 3 and data.size == lens.sum()
+    prefix = lens.astype(np.int64).ravel().cumsum().reshape(lens.shape)
+    for shift in range(4):                                                 # every alignment of the buffer
+        base = torch.zeros(data.size + shift, dtype=torch.uint8, device=DEV)
+        base[shift:] = torch.from_numpy(data).to(DEV)
+        out = torch.full((nl, nt, nc), 0xEE, dtype=torch.uint8, device=DEV)
+        tac.decode_fast_prefsum(torch.from_numpy(cdf.view(np.int16)).to(DEV), base[shift:],
+                                torch.from_numpy(prefix).to(DEV), out)
+        assert np.array_equal(out.cpu().numpy(), sym), shift

@@ -297,6 +297,15 @@ def main():
             "avg_launch_ms": round(dec_avg, 4),
         },
     }
+    # what one chunk weighs on the wire in the two flat containers (first chunk, vllm layout only)
+    if fmt == "vllm":
+        from cachegen_amd.serde import wire
+        flat_blob = wire.pack_chunks(enc, 0, 1)[0]
+        compact_blob = wire.pack_chunks(enc, 0, 1, compact=True)[0]
+        chunk_fp16 = 2 * L * min(chunk, T) * C * 2
+        result["first_chunk_container"] = {
+            "fp16_bytes": chunk_fp16, "flat_bytes": len(flat_blob), "compact_bytes": len(compact_blob),
+            "ratio_flat": round(chunk_fp16 / len(flat_blob), 3), "ratio_compact": round(chunk_fp16 / len(compact_blob), 3)}
     if chunk > 256:
         # streaming case: latency of decoding one chunk on its own
         tdim = 2 if fmt == "vllm" else 3

@@ -35,6 +35,7 @@
 #include "decoder.hpp"
 #include "scan_compact.hpp"
 #include "launch.hpp"
+#include "tables_wire.hpp"
 
 // ======================================================================================
 // C ABI
@@ -42,7 +43,7 @@
 extern "C" {
 
 const char *cg_last_error(void) { return g_error; }
-int cg_abi_version(void) { return 2; }
+int cg_abi_version(void) { return 3; }
 
 int64_t cg_num_chunks(int64_t T, int64_t chunk_tokens)
 {
@@ -331,6 +332,48 @@ int cg_decode_kv(const int16_t *cdf, int max_bins, const void *maxima, int max_d
     if (out_dt == CG_DT_BF16) CG_DISPATCH_BS(block, (launch_decode_kv_log2<BS, OUT_BF16>(a, grid, shmem, s)));
     else CG_DISPATCH_BS(block, (launch_decode_kv_log2<BS, OUT_F16>(a, grid, shmem, s)));
     return check_launch("decode_kv");
+}
+
+int cg_tables_to_counts(const int16_t *cdf, int max_bins, int64_t ngroups, int64_t C, const int32_t *tokens,
+                        uint8_t *counts, int32_t *nsym, int32_t *inexact, void *stream)
+{
+    if (!cdf || !tokens || !counts || !nsym || !inexact) return fail(CG_ERR_ARG, "tables_to_counts: null pointer");
+    if (int rc = check_lp(max_bins + 1, "tables_to_counts")) return rc;
+    if (ngroups <= 0 || C <= 0 || ngroups > 65535) return fail(CG_ERR_ARG, "tables_to_counts: bad group or channel count");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    clear_ints_kernel<<<dim3((unsigned)ceil_div(ngroups, kWireThreads)), dim3(kWireThreads), 0, s>>>(nsym, ngroups, inexact);
+    const dim3 grid((unsigned)ceil_div(C, kWireThreads), (unsigned)ngroups);
+    tables_to_counts_kernel<<<grid, dim3(kWireThreads), 0, s>>>(reinterpret_cast<const uint16_t *>(cdf), max_bins + 1, C,
+                                                               tokens, counts, nsym, inexact);
+    return check_launch("tables_to_counts");
+}
+
+int cg_pack_counts(const uint8_t *counts, int max_bins, int64_t ngroups, int64_t C, const int32_t *nsym,
+                   const int64_t *starts, uint8_t *out, void *stream)
+{
+    if (!counts || !nsym || !starts || !out) return fail(CG_ERR_ARG, "pack_counts: null pointer");
+    if (int rc = check_lp(max_bins + 1, "pack_counts")) return rc;
+    if (ngroups <= 0 || C <= 0 || ngroups > 65535) return fail(CG_ERR_ARG, "pack_counts: bad group or channel count");
+    const dim3 grid((unsigned)ceil_div(C, kWireThreads), (unsigned)ngroups);
+    pack_counts_kernel<<<grid, dim3(kWireThreads), 0, static_cast<hipStream_t>(stream)>>>(counts, max_bins + 1, C, nsym,
+                                                                                         starts, out);
+    return check_launch("pack_counts");
+}
+
+int cg_counts_to_tables(const uint8_t *data, int64_t data_bytes, int max_bins, int64_t ngroups, int64_t C,
+                        const int32_t *tokens, const uint8_t *nsym, const int64_t *starts, int16_t *cdf,
+                        int32_t *invalid, void *stream)
+{
+    if (!data || !tokens || !nsym || !starts || !cdf || !invalid) return fail(CG_ERR_ARG, "counts_to_tables: null pointer");
+    if (int rc = check_lp(max_bins + 1, "counts_to_tables")) return rc;
+    if (ngroups <= 0 || C <= 0 || ngroups > 65535 || data_bytes < 0)
+        return fail(CG_ERR_ARG, "counts_to_tables: bad group or channel count");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    clear_ints_kernel<<<dim3(1), dim3(kWireThreads), 0, s>>>(invalid, 1, nullptr);
+    const dim3 grid((unsigned)ceil_div(C, kWireThreads), (unsigned)ngroups);
+    counts_to_tables_kernel<<<grid, dim3(kWireThreads), 0, s>>>(data, data_bytes, max_bins + 1, C, tokens, nsym, starts,
+                                                               reinterpret_cast<uint16_t *>(cdf), invalid);
+    return check_launch("counts_to_tables");
 }
 
 }  // extern "C"

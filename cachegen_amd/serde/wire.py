@@ -266,53 +266,68 @@ def unpack_host(blob):
 # --------------------------------------------------------------------------- #
 # device form: one staging buffer, one copy over PCIe per direction
 # --------------------------------------------------------------------------- #
+def _stream():
+    import torch
+    return torch.cuda.current_stream().cuda_stream
+
+
 def _device_counts(cdf, tokens):
-    """Torch form of tables_to_counts + pack_counts for cdf int16 [nchunks, 2L, C, Lp] on the
-    device: (nsym uint8 [nchunks, 2L], count bytes uint8 [...]) or None."""
+    """Device form of tables_to_counts + pack_counts for cdf int16 [nchunks, 2L, C, Lp]:
+    (nsym list per (chunk, row), ragged count bytes uint8 on the device) or None if some table is
+    not the table of a histogram."""
     import torch
-    lp = cdf.shape[-1]
-    scale = 0xFFFF - (lp - 1)
+    from .. import _lib
+    nchunks, rows, C, lp = cdf.shape
+    G = nchunks * rows
     dev = cdf.device
-    n = torch.tensor(tokens, dtype=torch.int64, device=dev).view(-1, 1, 1, 1)
-    idx = torch.arange(lp, dtype=torch.int64, device=dev)
-    wide = cdf.to(torch.int64) & 0xFFFF
-    cum = ((wide - idx) * n + (scale - 1)) // scale
-    counts = cum[..., 1:] - cum[..., :-1]
-    rebuilt = (scale * cum) // n + idx
-    exact = bool(((cum[..., 0] == 0).all() & (counts >= 0).all() & (rebuilt == wide).all()).item())
-    if not exact:
-        return None
-    nsyms = lp - 1
-    used = counts.sum(dim=2) > 0
-    last = nsyms - torch.flip(used, dims=[-1]).to(torch.int64).argmax(dim=-1)
-    nsym = torch.where(used.any(-1), last, torch.ones_like(last))
-    mask = torch.arange(nsyms, device=dev).view(1, 1, 1, -1) < nsym[:, :, None, None]
-    data = counts.clamp(max=255).to(torch.uint8)[mask.expand_as(counts)]
-    return nsym.to(torch.uint8), data
+    cdf = cdf.contiguous()
+    tok = torch.tensor([t for t in tokens for _ in range(rows)], dtype=torch.int32, device=dev)
+    dense = torch.empty((G, C, lp - 1), dtype=torch.uint8, device=dev)
+    nsym = torch.empty(G, dtype=torch.int32, device=dev)
+    inexact = torch.empty(1, dtype=torch.int32, device=dev)
+    lib = _lib.lib()
+    with torch.cuda.device(dev):
+        _lib.check(lib.cg_tables_to_counts(cdf.data_ptr(), lp - 1, G, C, tok.data_ptr(), dense.data_ptr(),
+                                           nsym.data_ptr(), inexact.data_ptr(), _stream()))
+        host = torch.cat([nsym, inexact]).tolist()
+        if host[-1]:
+            return None
+        ks = host[:-1]
+        starts, total = [], 0
+        for k in ks:
+            starts.append(total)
+            total += C * k
+        data = torch.empty(total, dtype=torch.uint8, device=dev)
+        d_starts = torch.tensor(starts, dtype=torch.int64, device=dev)
+        _lib.check(lib.cg_pack_counts(dense.data_ptr(), lp - 1, G, C, nsym.data_ptr(), d_starts.data_ptr(),
+                                      data.data_ptr(), _stream()))
+    return ks, data
 
 
-def _device_tables(nsym, data, C, lp, tokens):
-    """Torch form of unpack_counts + counts_to_tables -> cdf int16 [nchunks, 2L, C, Lp]."""
+def _device_tables(nsym_host, nsym_dev, data, C, lp, tokens):
+    """Device form of unpack_counts + counts_to_tables -> cdf int16 [nchunks, 2L, C, Lp].
+    nsym_host: numpy uint8 [nchunks, 2L] (read from the blob on the host), nsym_dev the same bytes
+    on the device."""
     import torch
+    from .. import _lib
+    nchunks, rows = nsym_host.shape
+    G = nchunks * rows
     dev = data.device
-    nsyms = lp - 1
-    mask = (torch.arange(nsyms, device=dev).view(1, 1, 1, -1) < nsym[:, :, None, None].to(torch.int64))
-    mask = mask.expand(nsym.shape[0], nsym.shape[1], C, nsyms)
-    counts = torch.zeros(mask.shape, dtype=torch.int64, device=dev)
-    n = torch.tensor(tokens, dtype=torch.int64, device=dev).view(-1, 1, 1)
-    ok = int(mask.sum().item()) == data.numel()
-    if ok:
-        counts[mask] = data.to(torch.int64)
-        missing = n - counts.sum(-1)
-        fits = (missing == 0) | ((missing == 1) & ((counts == 255).sum(-1) == 1))
-        ok = bool(fits.all().item())
-    if not ok:
+    sizes = nsym_host.astype(np.int64).ravel() * C
+    starts = np.concatenate([[0], np.cumsum(sizes)[:-1]]).astype(np.int64)
+    if int(sizes.sum()) != data.numel():
+        raise ValueError("wire container: table section does not match its symbol counts")
+    small = torch.from_numpy(np.concatenate([starts, np.repeat(np.asarray(tokens, dtype=np.int64), rows)])).to(dev)
+    tok = small[G:].to(torch.int32)
+    cdf = torch.empty((nchunks, rows, C, lp), dtype=torch.int16, device=dev)
+    invalid = torch.empty(1, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().cg_counts_to_tables(data.data_ptr(), data.numel(), lp - 1, G, C, tok.data_ptr(),
+                                                  nsym_dev.data_ptr(), small.data_ptr(), cdf.data_ptr(),
+                                                  invalid.data_ptr(), _stream()))
+    if int(invalid.item()):
         raise ValueError("wire container: histogram counts do not add up to the chunk's tokens")
-    counts = counts + (counts == 255) * missing[..., None]
-    scale = 0xFFFF - nsyms
-    cum = torch.cat([torch.zeros_like(counts[..., :1]), counts.cumsum(-1)], dim=-1)
-    cdf = (scale * cum) // n[..., None] + torch.arange(lp, dtype=torch.int64, device=dev)
-    return cdf.to(torch.int16)          # wraps values >= 32768 to their int16 bit pattern
+    return cdf
 
 
 def pack_chunks(enc, first_chunk: int = 0, num_chunks: Optional[int] = None, per_chunk: bool = True,
@@ -345,11 +360,11 @@ def pack_chunks(enc, first_chunk: int = 0, num_chunks: Optional[int] = None, per
         if S <= MAX_STREAM_BYTES:
             got = _device_counts(enc.cdf[c0:c1], all_tokens[c0:c1])
             if got is not None:
-                nsym, data = got
-                per_chunk_bytes = (nsym.to(torch.int64).sum(dim=1) * C).tolist()
+                ks, data = got                                   # nsym per (chunk, row), ragged count bytes
                 starts = [0]
-                for b in per_chunk_bytes:
-                    starts.append(starts[-1] + b)
+                for k in range(c1 - c0):
+                    starts.append(starts[-1] + C * sum(ks[k * 2 * L:(k + 1) * 2 * L]))
+                nsym = torch.tensor(ks, dtype=torch.uint8, device=data.device).view(c1 - c0, 2 * L)
                 packed = (nsym, data, starts)
                 flags |= FLAG_COUNT_TABLES
         lo, hi = torch.stack([enc.lengths.min(), enc.lengths.max()]).tolist()
@@ -420,11 +435,12 @@ def unpack_to_device(blob, device):
         raw = section("cdf", torch.uint8, (-1,))
         if raw.numel() < nchunks * 2 * L:
             raise ValueError("wire container: table section does not match its symbol counts")
-        nsym = raw[:nchunks * 2 * L].view(nchunks, 2 * L)
-        lo, hi = torch.stack([nsym.min(), nsym.max()]).tolist()
-        if lo < 1 or hi > lp - 1:
+        off = geo["cdf"][0]
+        nsym_host = np.frombuffer(blob, dtype=np.uint8, count=nchunks * 2 * L, offset=off).reshape(nchunks, 2 * L)
+        if int(nsym_host.min()) < 1 or int(nsym_host.max()) > lp - 1:
             raise ValueError("wire container: symbol count outside the table")
-        cdf = _device_tables(nsym, raw[nchunks * 2 * L:], C, lp, chunk_token_counts(T, h["chunk_tokens"]))
+        cdf = _device_tables(nsym_host, raw[:nchunks * 2 * L], raw[nchunks * 2 * L:], C, lp,
+                             chunk_token_counts(T, h["chunk_tokens"]))
     else:
         cdf = section("cdf", torch.int16, (nchunks, 2 * L, C, lp))
     maxima = section("maxima", torch.bfloat16 if h["bf16_maxima"] else torch.float16, (2, L, T))

@@ -170,6 +170,35 @@ int cg_decode_kv(const int16_t *cdf, int max_bins, const void *maxima, int max_d
                  void *out, int out_dt, int64_t ol, int64_t okv, int64_t ot, int64_t oh,
                  void *stream);
 
+/* ---------------------------------------------------------------------------
+ * Tables as histogram counts, for containers that store the counts (no counterpart in
+ * the reference, whose container pickles the tables; the relation inverted here is
+ * cal_cdf.cu:29-49).  A group is one (chunk, row): C channels sharing a token count
+ * tokens[g] <= 256.
+ * ------------------------------------------------------------------------- */
+
+/* cdf     device int16 [ngroups, C, max_bins+1]
+ * tokens  device int32 [ngroups]: tokens the tables of group g were built over (1..256)
+ * counts  device uint8 [ngroups, C, max_bins], written: histogram counts, 256 stored as 255
+ * nsym    device int32 [ngroups], written: 1 + the largest symbol that occurs in the group
+ * inexact device int32 [1], written: 1 if some table is not the table of any histogram */
+int cg_tables_to_counts(const int16_t *cdf, int max_bins, int64_t ngroups, int64_t C,
+                        const int32_t *tokens, uint8_t *counts, int32_t *nsym, int32_t *inexact,
+                        void *stream);
+
+/* Ragged form of `counts`: out[starts[g] + ch*nsym[g] + j] = counts[g, ch, j], j < nsym[g]. */
+int cg_pack_counts(const uint8_t *counts, int max_bins, int64_t ngroups, int64_t C,
+                   const int32_t *nsym, const int64_t *starts, uint8_t *out, void *stream);
+
+/* Ragged counts back to tables.
+ * data    device uint8 [data_bytes]: as written by cg_pack_counts (never read outside)
+ * nsym    device uint8 [ngroups]; starts device int64 [ngroups]
+ * cdf     device int16 [ngroups, C, max_bins+1], written
+ * invalid device int32 [1], written: 1 if some channel's counts do not add up to tokens[g] */
+int cg_counts_to_tables(const uint8_t *data, int64_t data_bytes, int max_bins, int64_t ngroups, int64_t C,
+                        const int32_t *tokens, const uint8_t *nsym, const int64_t *starts, int16_t *cdf,
+                        int32_t *invalid, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

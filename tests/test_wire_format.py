@@ -285,3 +285,28 @@ def test_compact_serde_decodes_like_the_pickle_serde():
             if ntok <= 256:
                 assert len(b) < 0.75 * len(a)
             assert torch.equal(d.from_bytes(a), d.from_bytes(b))
+
+
+@pytest.mark.gpu
+def test_corrupt_compact_blob_is_rejected_on_the_device():
+    from cachegen_amd import codec
+    from cachegen_amd.kvgen import make_kv
+    kv = make_kv(2, 256, 2, 64, seed=3, device=DEV)
+    bins = torch.tensor([32.0, 16.0])
+    enc = codec.encode_kv(kv, bins, bins, chunk_tokens=256)
+    blob = wire.pack_chunks(enc, compact=True)[0]
+    h = wire.read_header(blob)
+    assert h["count_tables"]
+    off = h["geometry"]["cdf"][0]
+    bad = bytearray(blob)
+    bad[off + 4 + 7] = (bad[off + 4 + 7] + 1) % 200        # one histogram count (4 bytes of nsym come first)
+    with pytest.raises(ValueError, match="add up"):
+        wire.unpack_to_device(bytes(bad), DEV)
+    bad = bytearray(blob)
+    bad[off] = 200                                         # a symbol count beyond the table
+    with pytest.raises(ValueError, match="outside the table"):
+        wire.unpack_to_device(bytes(bad), DEV)
+    bad = bytearray(blob)
+    bad[off] = max(1, bad[off] - 1)                        # a symbol count that no longer matches the section size
+    with pytest.raises(ValueError, match="does not match"):
+        wire.unpack_to_device(bytes(bad), DEV)

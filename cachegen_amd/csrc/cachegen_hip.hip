@@ -186,7 +186,10 @@ size_t cg_encode_kv_workspace(int64_t L, int64_t T, int64_t C, int64_t chunk_tok
     size_t total = align_up((size_t)nstreams * kSub, 256);        // symbols: a 256-token slot per stream
     total += (size_t)ceil_div(nstreams, kSlotTile) * kSlotTile * kStreamCap;   // encoder scratch: whole tiles of slots
     total += cg_scan_workspace(nstreams);
-    total += align_up((size_t)ceil_div(nstreams, kSlotTile) * sizeof(int64_t), 256);   // bytes per tile of streams
+    const int64_t ntiles = ceil_div(nstreams, kSlotTile);
+    total += align_up((size_t)ntiles * sizeof(int32_t), 256);          // bytes per tile of streams
+    total += align_up((size_t)(ntiles + 1) * sizeof(int64_t), 256);    // their running sums
+    total += cg_scan_workspace(ntiles);
     return total;
 }
 
@@ -219,7 +222,12 @@ int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int
     ws += (size_t)ceil_div(nstreams, kSlotTile) * kSlotTile * kStreamCap;
     void *scan_scratch = ws;
     ws += cg_scan_workspace(nstreams);
-    int64_t *tile_sums = reinterpret_cast<int64_t *>(ws);
+    const int64_t ntiles = ceil_div(nstreams, kSlotTile);
+    int32_t *tile_sums = reinterpret_cast<int32_t *>(ws);
+    ws += align_up((size_t)ntiles * sizeof(int32_t), 256);
+    int64_t *tile_base = reinterpret_cast<int64_t *>(ws);
+    ws += align_up((size_t)(ntiles + 1) * sizeof(int64_t), 256);
+    void *tile_scan_scratch = ws;
     uint16_t *tables = reinterpret_cast<uint16_t *>(cdf);
 
     clear_status_kernel<<<1, 1, 0, s>>>(status);
@@ -278,9 +286,9 @@ int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int
     if (cblocks > INT_MAX) return fail(CG_ERR_ARG, "encode_kv: too many streams");
     const int32_t skew = (int32_t)(reinterpret_cast<uintptr_t>(payload) & 3u);
     if (fused_scan) {
-        scan_sums_kernel<<<dim3(1), dim3(kScanThreads), 0, s>>>(tile_sums, cblocks);
+        if (int rc = launch_scan(tile_sums, cblocks, INT_MAX, tile_base, tile_scan_scratch, s)) return rc;
         compact_streams_kernel<true><<<dim3((unsigned)cblocks), dim3(256), 0, s>>>(
-            scratch, kStreamCap, offsets, lengths, tile_sums, nstreams, payload, payload_cap, skew, status);
+            scratch, kStreamCap, offsets, lengths, tile_base, nstreams, payload, payload_cap, skew, status);
     } else {
         if (int rc = launch_scan(lengths, nstreams, kStreamCap, offsets, scan_scratch, s)) return rc;
         compact_streams_kernel<false><<<dim3((unsigned)cblocks), dim3(256), 0, s>>>(

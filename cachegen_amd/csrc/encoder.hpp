@@ -200,7 +200,7 @@ struct EncodeArgs {
     int32_t cap;
     int32_t *lengths;       // [sub][row][channel]
     int32_t *status;        // may be null
-    int64_t *tile_sums;     // SLOTS, one block per tile of kSlotTile streams: stored bytes per tile, or null
+    int32_t *tile_sums;     // SLOTS, one block per tile of kSlotTile streams: stored bytes per tile, or null
     const float *key_bins, *value_bins;     // float32 [L] each, or null when the levels are not known
     int64_t L;
     StreamGrid sg;
@@ -347,9 +347,9 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
         if ((tid & 63) == 0) wave_sums[tid >> 6] = v;
         __syncthreads();
         if (tid == 0) {
-            int64_t total = 0;
+            int32_t total = 0;
             for (int w = 0; w < BS / 64; ++w) total += wave_sums[w];
-            a.tile_sums[blockIdx.x] = total;
+            a.tile_sums[blockIdx.x] = total;                  // at most 256 streams of 256 bytes
         }
     }
 }

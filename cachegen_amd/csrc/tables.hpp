@@ -137,8 +137,16 @@ __global__ __launch_bounds__(BS) void calculate_cdf_kernel(CdfArgs a)
     const int64_t row = b % a.rows;
     const int64_t chunk = b / a.rows;
     const int64_t ch = (int64_t)ctile * BS + tid;
+    // byte symbols: one 32-bit counter per (entry, lane); packed symbols (the fused path, whose
+    // symbols all lie inside the table): 16-bit counters, two lanes to a word, as in the encoder
     uint32_t *col = smem + tid;
-    for (int i = 0; i < lp; ++i) col[i * BS] = 0;
+    uint16_t *tab16 = reinterpret_cast<uint16_t *>(smem);
+    if (PACKED) {
+        for (int i = 0; i < lp; ++i) tab16[i * BS + tid] = 0;
+        __syncthreads();                     // a lane's neighbour shares its words
+    } else {
+        for (int i = 0; i < lp; ++i) col[i * BS] = 0;
+    }
 
     const int64_t t0 = chunk * a.g.S;
     int64_t t1 = t0 + a.g.S;
@@ -161,6 +169,8 @@ __global__ __launch_bounds__(BS) void calculate_cdf_kernel(CdfArgs a)
                 if (v < mb) atomicAdd(col + (v + 1) * BS, 1u);
             }
         } else {
+            uint32_t *const pair = smem + (tid >> 1);
+            const uint32_t one = (tid & 1) ? 0x10000u : 1u;
             const int64_t sub0 = chunk * a.g.nsc;
             const int nsubs = (int)((t1 - t0 + kSub - 1) / kSub);
             for (int sidx = 0; sidx < nsubs; ++sidx) {
@@ -168,23 +178,33 @@ __global__ __launch_bounds__(BS) void calculate_cdf_kernel(CdfArgs a)
                 const int n = left < kSub ? (int)left : kSub;
                 const uint32_t *wp = a.sym4 + ((row * a.nsub + sub0 + sidx) * kWordsPerSub) * a.nc + ch;
                 const int nwords = (n + 3) >> 2;
-                for (int w0 = 0; w0 < nwords; w0 += 4) {
-                    uint32_t v[4];
+                constexpr int kBatch = 16;          // words in flight per lane
+                for (int w0 = 0; w0 < nwords; w0 += kBatch) {
+                    uint32_t v[kBatch];
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) v[j] = (w0 + j < nwords) ? wp[(int64_t)(w0 + j) * a.nc] : 0u;
+                    for (int j = 0; j < kBatch; ++j) v[j] = (w0 + j < nwords) ? wp[(int64_t)(w0 + j) * a.nc] : 0u;
 #pragma unroll
-                    for (int j = 0; j < 16; ++j) {
-                        const uint32_t s = (v[j >> 2] >> (8 * (j & 3))) & 0xFFu;
-                        if (w0 * 4 + j < n && s < mb) atomicAdd(col + (s + 1) * BS, 1u);
+                    for (int j = 0; j < 4 * kBatch; ++j) {
+                        uint32_t s = (v[j >> 2] >> (8 * (j & 3))) & 0xFFu;
+                        s = s < mb - 1u ? s : mb - 1u;
+                        if (w0 * 4 + j < n) atomicAdd(pair + (s + 1) * (BS / 2), one);
                     }
                 }
             }
         }
-        normalize_column<BS>(col, lp, a.max_bins);
+        if (!PACKED) normalize_column<BS>(col, lp, a.max_bins);
     }
-    __syncthreads();
     const int64_t ch0 = (int64_t)ctile * BS;
-    write_tables<BS>(smem, a.cdf + ((chunk * a.rows + row) * a.nc + ch0) * lp, lp, ch0, a.nc);
+    uint16_t *dst = a.cdf + ((chunk * a.rows + row) * a.nc + ch0) * lp;
+    if (PACKED) {
+        __syncthreads();                     // the neighbour's atomics on the shared words are done
+        if (ch < a.nc) normalize_column16<BS>(tab16 + tid, lp, a.max_bins, (uint32_t)(t1 - t0));
+        __syncthreads();
+        write_tables16<BS>(tab16, dst, lp, ch0, a.nc);
+    } else {
+        __syncthreads();
+        write_tables<BS>(smem, dst, lp, ch0, a.nc);
+    }
 }
 
 // ------------------------------------------------------------------------------------

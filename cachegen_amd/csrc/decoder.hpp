@@ -292,10 +292,9 @@ __global__ __launch_bounds__(BS) void decode_streams_kernel(DecodeArgs a)
         const uint16_t *src = a.cdf + ((id.chunk * a.sg.rows + id.row) * a.sg.nc + ch0) * lp;
         const int64_t nvalid = (a.sg.nc - ch0 < BS) ? (a.sg.nc - ch0) : BS;
         const int total = (int)nvalid * lp;
-        for (int i = tid; i < total; i += BS) {
-            const int c = i / lp, e = i - c * lp;
-            *reinterpret_cast<uint16_t *>(rows + e * kRow + 2 * c) = e == 0 ? (uint16_t)0 : src[i];
-        }
+        TableWalk w(tid, BS, lp);
+        for (int i = tid; i < total; i += BS, w.next(lp))
+            *reinterpret_cast<uint16_t *>(rows + w.e * kRow + 2 * w.c) = w.e == 0 ? (uint16_t)0 : src[i];
     }
     int64_t kvi = 0, l = 0;
     int special = 0;                   // a row maximum that is infinite or NaN

@@ -20,6 +20,28 @@ namespace {
 // counters, and the block writes its tables back transposed so stores coalesce.
 // ------------------------------------------------------------------------------------
 
+// Walks i = start, start + step, ... over tables stored one after the other ([channel][lp]) and
+// keeps (c, e) = (i / lp, i % lp) up to date with one divide at the start instead of one per step.
+struct TableWalk {
+    int c, e, dc, de;
+    __device__ __forceinline__ TableWalk(int start, int step, int lp)
+    {
+        c = start / lp;
+        e = start - c * lp;
+        dc = step / lp;
+        de = step - dc * lp;
+    }
+    __device__ __forceinline__ void next(int lp)
+    {
+        c += dc;
+        e += de;
+        if (e >= lp) {
+            e -= lp;
+            ++c;
+        }
+    }
+};
+
 // Running sum and normalisation of one lane's column col[i * BS], i in [0, lp).
 template <int BS>
 __device__ __forceinline__ void normalize_column(uint32_t *col, int lp, int max_bins)
@@ -42,9 +64,9 @@ __device__ __forceinline__ void write_tables(const uint32_t *tab, uint16_t *cdf,
 {
     const int64_t nvalid = (nc - ch0 < BS) ? (nc - ch0) : BS;
     const int total = (int)nvalid * lp;
-    for (int i = threadIdx.x; i < total; i += BS) {
-        const int c = i / lp, e = i - c * lp;
-        cdf[i] = (uint16_t)tab[e * BS + c];
+    TableWalk w(threadIdx.x, BS, lp);
+    for (int i = threadIdx.x; i < total; i += BS, w.next(lp)) {
+        cdf[i] = (uint16_t)tab[w.e * BS + w.c];
     }
 }
 
@@ -54,9 +76,9 @@ __device__ __forceinline__ void stage_tables(uint32_t *tab, const uint16_t *cdf,
 {
     const int64_t nvalid = (nc - ch0 < BS) ? (nc - ch0) : BS;
     const int total = (int)nvalid * lp;
-    for (int i = threadIdx.x; i < total; i += BS) {
-        const int c = i / lp, e = i - c * lp;
-        tab[e * BS + c] = cdf[i];
+    TableWalk w(threadIdx.x, BS, lp);
+    for (int i = threadIdx.x; i < total; i += BS, w.next(lp)) {
+        tab[w.e * BS + w.c] = cdf[i];
     }
 }
 
@@ -68,9 +90,9 @@ __device__ __forceinline__ void stage_tables16(uint16_t *tab, const uint16_t *cd
 {
     const int64_t nvalid = (nc - ch0 < BS) ? (nc - ch0) : BS;
     const int total = (int)nvalid * lp;
-    for (int i = threadIdx.x; i < total; i += BS) {
-        const int c = i / lp, e = i - c * lp;
-        tab[e * BS + c] = cdf[i];
+    TableWalk w(threadIdx.x, BS, lp);
+    for (int i = threadIdx.x; i < total; i += BS, w.next(lp)) {
+        tab[w.e * BS + w.c] = cdf[i];
     }
 }
 
@@ -79,9 +101,9 @@ __device__ __forceinline__ void write_tables16(const uint16_t *tab, uint16_t *cd
 {
     const int64_t nvalid = (nc - ch0 < BS) ? (nc - ch0) : BS;
     const int total = (int)nvalid * lp;
-    for (int i = threadIdx.x; i < total; i += BS) {
-        const int c = i / lp, e = i - c * lp;
-        cdf[i] = tab[e * BS + c];
+    TableWalk w(threadIdx.x, BS, lp);
+    for (int i = threadIdx.x; i < total; i += BS, w.next(lp)) {
+        cdf[i] = tab[w.e * BS + w.c];
     }
 }
 

@@ -98,7 +98,7 @@ int cg_encode_fast_new(const int16_t *cdf, int lp, const int8_t *sym, int64_t nl
     // nt == 0 still writes the two closing bits of every stream
     if (int rc = make_grid(nl, nc, nt ? nt : 1, nt ? nt : 1, 1, block, a.sg, nblocks)) return rc;
     if (nt == 0) a.sg.g.T = 0;
-    const size_t shmem = (size_t)lp * block * sizeof(uint16_t);
+    const size_t shmem = (size_t)lp * (block + 2) * sizeof(uint16_t);      // TableStride<BS>::k16 per entry
     const bool aligned = aligned_to(out, 4) && o0 % 4 == 0 && o1 % 4 == 0;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const dim3 grid((unsigned)nblocks), blk(block);
@@ -247,7 +247,7 @@ int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int
     a.L = L;
     int64_t nblocks;
     if (int rc = make_grid(rows, C, T, chunk_tokens, nsub, block, a.sg, nblocks)) return rc;
-    const size_t shmem = (size_t)lp * block * sizeof(uint16_t);
+    const size_t shmem = (size_t)lp * (block + 2) * sizeof(uint16_t);      // TableStride<BS>::k16 per entry
     const dim3 grid((unsigned)nblocks), blk(block);
     // when every encoder block is exactly one tile of the scratch, the blocks leave their byte
     // counts behind and the compaction computes the stream offsets itself

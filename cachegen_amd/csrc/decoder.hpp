@@ -146,11 +146,17 @@ struct DecodeLane {
     uint32_t off, low, span;
     lds_char *colp;            // this lane's entry 0
     int lutoff;                // from an entry of this lane to its row's quotient
+    // the entries the first two probes of the unrolled search look at (one for the first, one
+    // of two for the second), read once per stream: two LDS round trips less per symbol
+    uint32_t probe1, probe2_lo, probe2_hi;
     uint8_t *osym;
     uint16_t *okv;
     float anchor;              // reconstructed anchor row value (delta mode)
     int phase;                 // position of the token inside its group (delta mode)
 };
+
+// Distance of the unrolled search's first probe from entry 0, in entries.
+__host__ __device__ constexpr int first_probe(int log2, int skip) { return log2 >= 2 ? ((1 << log2) >> 1) >> skip : 0; }
 
 // One symbol.  SKIP: how many of the search's first probes are left out because the row's
 // alphabet fits the lower 2^(LOG2-SKIP) entries.  SAFE: the last table entry may be decoded
@@ -160,64 +166,77 @@ __device__ __forceinline__ void decode_symbol(const DecodeArgs &a, DecodeLane &s
                                               float rm, int i, bool last_symbol)
 {
     constexpr int kRow = DecodeLayout<BS, OUT>::kRow;
+    constexpr int kStep1 = first_probe(LOG2, SKIP), kStep2 = kStep1 >> 1;
     lds_char *p = s.colp;              // entry of the decoded symbol
     lds_char *const plast = s.colp + (lp - 2) * kRow;
     uint32_t t_lo, width;
-    if (__builtin_expect(s.span == 0, 0)) {
-        // full range: T(m) = cdf[m] << 16, so compare table values with off >> 16
+    float q = 0.0f;                    // (symbol - C) / C
+    const bool full_range = s.span == 0;
+    const uint32_t sh = s.span >> 16, sl = s.span & 0xFFFFu;
+    if (LOG2 >= 2 && __builtin_expect(full_range, 0)) {
+        // full range (a stream's first symbol, hardly ever later): T(m) = cdf[m] << 16, so
+        // table values are compared with off >> 16
         const uint32_t key = s.off >> 16;
-        if (LOG2 >= 0) {
 #pragma unroll
-            for (int step = ((1 << LOG2) >> 1) >> SKIP; step >= 1; step >>= 1)
-                p = (lds_entry(p, step * kRow) <= key) ? p + step * kRow : p;
-        } else {
-            int lo_i = 0, hi_i = lp - 1;
-            for (int step = 0; step < nsteps; ++step) {
-                const int mid = (lo_i + hi_i) >> 1;
-                const bool le = mid > 0 && lds_entry(s.colp, mid * kRow) <= key;
-                lo_i = le ? mid : lo_i;
-                hi_i = le ? hi_i : mid;
-            }
-            p = s.colp + lo_i * kRow;
-        }
+        for (int step = kStep1; step >= 1; step >>= 1)
+            p = (lds_entry(p, step * kRow) <= key) ? p + step * kRow : p;
         const uint32_t c_lo = lds_entry(p, 0);
         const uint32_t c_hi = (SAFE && p == plast) ? 0x10000u : lds_entry(p, kRow);
+        if (OUT != OUT_SYMBOLS) q = *(lds_f32 *)(p + s.lutoff);
         t_lo = c_lo << 16;
         width = (c_hi - c_lo) << 16;
-    } else {
-        const uint32_t sh = s.span >> 16, sl = s.span & 0xFFFFu;
-        if (LOG2 >= 0) {
-            // probe with the lower bound sh * c <= T(c); it can only overshoot
-#pragma unroll
-            for (int step = ((1 << LOG2) >> 1) >> SKIP; step >= 1; step >>= 1) {
-                const uint32_t t = mul24(sh, lds_entry(p, step * kRow));
-                p = (t <= s.off) ? p + step * kRow : p;
-            }
-            t_lo = scale_span(sh, sl, lds_entry(p, 0));
-            // entry 0 is 0 (forced when the tables are staged), so this stops there at the latest
-            while (__builtin_expect(t_lo > s.off, 0)) {
-                p -= kRow;
-                t_lo = scale_span(sh, sl, lds_entry(p, 0));
-            }
-        } else {
-            int lo_i = 0, hi_i = lp - 1;
-            for (int step = 0; step < nsteps; ++step) {
-                const int mid = (lo_i + hi_i) >> 1;
-                const uint32_t t = scale_span(sh, sl, lds_entry(s.colp, mid * kRow));
-                const bool le = mid > 0 && t <= s.off;
-                lo_i = le ? mid : lo_i;
-                hi_i = le ? hi_i : mid;
-            }
-            p = s.colp + lo_i * kRow;
-            t_lo = scale_span(sh, sl, lds_entry(p, 0));
+    } else if (LOG2 >= 2) {
+        // largest m with T(m) <= off, probed with the lower bound sh * c <= T(c), which can
+        // only overshoot; the first two probes compare entries held in registers
+        const bool up1 = mul24(sh, s.probe1) <= s.off;
+        p = up1 ? p + kStep1 * kRow : p;
+        if (kStep2 >= 1) {
+            const uint32_t c2 = up1 ? s.probe2_hi : s.probe2_lo;
+            p = (mul24(sh, c2) <= s.off) ? p + kStep2 * kRow : p;
         }
-        const uint32_t c_hi = (SAFE && p == plast) ? 0x10000u : lds_entry(p, kRow);
+#pragma unroll
+        for (int step = kStep2 >> 1; step >= 1; step >>= 1)
+            p = (mul24(sh, lds_entry(p, step * kRow)) <= s.off) ? p + step * kRow : p;
+        // both bounds and the quotient in one round trip (entry lp - 1 exists, so the upper
+        // bound of the last symbol can be read and then replaced)
+        uint32_t c_lo = lds_entry(p, 0);
+        uint32_t c_hi = lds_entry(p, kRow);
+        if (OUT != OUT_SYMBOLS) q = *(lds_f32 *)(p + s.lutoff);
+        t_lo = scale_span(sh, sl, c_lo);
+        // entry 0 is 0 (forced when the tables are staged), so this stops there at the latest
+        while (__builtin_expect(t_lo > s.off, 0)) {
+            p -= kRow;
+            c_hi = c_lo;
+            c_lo = lds_entry(p, 0);
+            if (OUT != OUT_SYMBOLS) q = *(lds_f32 *)(p + s.lutoff);
+            t_lo = scale_span(sh, sl, c_lo);
+        }
+        if (SAFE && p == plast) c_hi = 0x10000u;                                // dec_new.cu:278
         width = scale_span(sh, sl, c_hi) - t_lo;
+    } else {
+        int lo_i = 0, hi_i = lp - 1;
+        for (int step = 0; step < nsteps; ++step) {
+            const int mid = (lo_i + hi_i) >> 1;
+            const uint32_t c = lds_entry(s.colp, mid * kRow);
+            const bool le = mid > 0 && (full_range ? c <= (s.off >> 16) : scale_span(sh, sl, c) <= s.off);
+            lo_i = le ? mid : lo_i;
+            hi_i = le ? hi_i : mid;
+        }
+        p = s.colp + lo_i * kRow;
+        const uint32_t c_lo = lds_entry(p, 0);
+        const uint32_t c_hi = (SAFE && p == plast) ? 0x10000u : lds_entry(p, kRow);
+        if (OUT != OUT_SYMBOLS) q = *(lds_f32 *)(p + s.lutoff);
+        if (full_range) {
+            t_lo = c_lo << 16;
+            width = (c_hi - c_lo) << 16;
+        } else {
+            t_lo = scale_span(sh, sl, c_lo);
+            width = scale_span(sh, sl, c_hi) - t_lo;
+        }
     }
     if (OUT == OUT_SYMBOLS) {
         s.osym[(int64_t)i * a.o1] = (uint8_t)((uint32_t)(p - s.colp) / (uint32_t)kRow);
     } else {
-        const float q = *(lds_f32 *)(p + s.lutoff);
         float v = __fmul_rn(q, rm);
         // the product is rounded to float32 before it is rounded to 16 bits (decoder.py:28-34
         // works in float32): keep the compiler from merging the two into one mixed-precision
@@ -255,6 +274,13 @@ __device__ __forceinline__ void decode_lane(const DecodeArgs &a, DecodeLane &s, 
     int nsteps = 0;
     if (LOG2 < 0)
         while ((1 << nsteps) < lp - 1) ++nsteps;
+    if (LOG2 >= 2) {
+        constexpr int kRow = DecodeLayout<BS, OUT>::kRow;
+        constexpr int kStep1 = first_probe(LOG2, SKIP), kStep2 = kStep1 >> 1;
+        s.probe1 = lds_entry(s.colp, kStep1 * kRow);
+        s.probe2_lo = lds_entry(s.colp, kStep2 * kRow);
+        s.probe2_hi = lds_entry(s.colp, (kStep1 + kStep2) * kRow);
+    }
     for (int i0 = 0; i0 < n; i0 += 4, rmp += 4) {
         // the maxima of the next four token rows (the array is padded to a multiple of four)
         float rm[4] = {0.0f, 0.0f, 0.0f, 0.0f};

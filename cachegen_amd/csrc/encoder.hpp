@@ -116,7 +116,7 @@ struct BitWriter {
 // span to span << n for E1/E2 and E3 steps alike.
 template <int BS, bool ALIGNED>
 struct RangeEncoder {
-    const uint16_t *col;    // this lane's table column: entry e at col[e * BS]
+    const uint16_t *col;    // this lane's table column: entry e at col[e * TableStride<BS>::k16]
     uint32_t smax;          // lp - 2: the largest symbol
     uint32_t low, span, pend;
     BitWriter<ALIGNED> w;
@@ -143,8 +143,9 @@ struct RangeEncoder {
     __device__ __forceinline__ void put_symbol(uint32_t s)
     {
         s = s < smax ? s : smax;                        // keep table reads inside the table
-        const uint32_t c_lo = col[s * BS];
-        const uint32_t c_next = col[s * BS + BS];
+        constexpr int kS = TableStride<BS>::k16;
+        const uint32_t c_lo = col[s * kS];
+        const uint32_t c_next = col[s * kS + kS];
         const uint32_t c_hi = (SENTINEL && s == smax) ? 0x10000u : c_next;
         uint32_t t_lo, width;
         if (__builtin_expect(span == 0, 0)) {
@@ -242,7 +243,7 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
     };
 
     if (FUSE_CDF) {
-        for (int i = 0; i < lp; ++i) col[i * BS] = 0;
+        for (int i = 0; i < lp; ++i) col[i * TableStride<BS>::k16] = 0;
         if (id.active) {
             const uint32_t smax = (uint32_t)(lp - 2);
             // two lanes share a 32-bit LDS word: each adds to its own half with one atomic that
@@ -259,7 +260,7 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
                     for (int j = 0; j < 4; ++j) {
                         uint32_t s = (v >> (8 * j)) & 0xFFu;
                         s = s < smax ? s : smax;
-                        if ((h * 32 + w) * 4 + j < id.n) atomicAdd(pair + (s + 1) * (BS / 2), one);
+                        if ((h * 32 + w) * 4 + j < id.n) atomicAdd(pair + (s + 1) * (TableStride<BS>::k16 / 2), one);
                     }
                 }
             }

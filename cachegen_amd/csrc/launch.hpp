@@ -50,7 +50,8 @@ int launch_cdf(const uint8_t *sym, const uint32_t *sym4, int64_t nsub, int64_t r
                int64_t nc, int64_t s0, int64_t s1, int64_t s2, int max_bins, int64_t S,
                uint16_t *cdf, hipStream_t stream)
 {
-    const int block = pick_block(nc, max_bins + 1);
+    int block = pick_block(nc, max_bins + 1);
+    while (!sym4 && block > 64 && (size_t)(max_bins + 1) * (block + 1) * sizeof(uint32_t) > 64 * 1024) block /= 2;
     CdfArgs a;
     a.sym = sym;
     a.s0 = s0;
@@ -68,7 +69,8 @@ int launch_cdf(const uint8_t *sym, const uint32_t *sym4, int64_t nsub, int64_t r
     a.g.nsc = (int32_t)ceil_div(S, kSub);
     const int64_t nblocks = ceil_div(T, S) * rows * a.ctiles;
     if (nblocks <= 0 || nblocks > INT_MAX) return fail(CG_ERR_ARG, "calculate_cdf: grid out of range");
-    const size_t shmem = (size_t)(max_bins + 1) * block * (sym4 ? sizeof(uint16_t) : sizeof(uint32_t));
+    const size_t shmem = sym4 ? (size_t)(max_bins + 1) * (block + 2) * sizeof(uint16_t)
+                              : (size_t)(max_bins + 1) * (block + 1) * sizeof(uint32_t);     // TableStride
     const dim3 grid((unsigned)nblocks), blk(block);
     if (sym4) CG_DISPATCH_BS(block, (calculate_cdf_kernel<BS, true><<<grid, blk, shmem, stream>>>(a)));
     else CG_DISPATCH_BS(block, (calculate_cdf_kernel<BS, false><<<grid, blk, shmem, stream>>>(a)));

@@ -20,6 +20,16 @@ namespace {
 // counters, and the block writes its tables back transposed so stores coalesce.
 // ------------------------------------------------------------------------------------
 
+// Row strides of the per-block tables in LDS (entry e of lane c is element e * stride + c).  One
+// more than a multiple of 64 banks' worth: the block reads and writes its tables transposed
+// (consecutive lanes take consecutive entries of one channel), and with a stride of exactly
+// BS elements every lane of a wavefront would hit the same bank.
+template <int BS>
+struct TableStride {
+    static constexpr int k16 = BS + 2;      // 16-bit entries: BS/2 + 1 words
+    static constexpr int k32 = BS + 1;      // 32-bit entries
+};
+
 // Walks i = start, start + step, ... over tables stored one after the other ([channel][lp]) and
 // keeps (c, e) = (i / lp, i % lp) up to date with one divide at the start instead of one per step.
 struct TableWalk {
@@ -42,23 +52,24 @@ struct TableWalk {
     }
 };
 
-// Running sum and normalisation of one lane's column col[i * BS], i in [0, lp).
+// Running sum and normalisation of one lane's column col[i * stride], i in [0, lp).
 template <int BS>
 __device__ __forceinline__ void normalize_column(uint32_t *col, int lp, int max_bins)
 {
+    constexpr int kS = TableStride<BS>::k32;
     uint32_t running = 0;
     for (int i = 1; i < lp; ++i) {
-        running = (running + col[i * BS]) & 0xFFFFu;
-        col[i * BS] = running;
+        running = (running + col[i * kS]) & 0xFFFFu;
+        col[i * kS] = running;
     }
     const uint32_t scale = 0xFFFFu - (uint32_t)max_bins;
     for (int i = 0; i < lp; ++i) {
-        const uint32_t q = running ? (scale * col[i * BS] / running) & 0xFFFFu : 0u;
-        col[i * BS] = (q + (uint32_t)i) & 0xFFFFu;
+        const uint32_t q = running ? (scale * col[i * kS] / running) & 0xFFFFu : 0u;
+        col[i * kS] = (q + (uint32_t)i) & 0xFFFFu;
     }
 }
 
-// Write the block's tables tab[entry * BS + lane] to cdf[lane][entry], coalesced.
+// Write the block's tables tab[entry * stride + lane] to cdf[lane][entry], coalesced.
 template <int BS>
 __device__ __forceinline__ void write_tables(const uint32_t *tab, uint16_t *cdf, int lp, int64_t ch0, int64_t nc)
 {
@@ -66,11 +77,11 @@ __device__ __forceinline__ void write_tables(const uint32_t *tab, uint16_t *cdf,
     const int total = (int)nvalid * lp;
     TableWalk w(threadIdx.x, BS, lp);
     for (int i = threadIdx.x; i < total; i += BS, w.next(lp)) {
-        cdf[i] = (uint16_t)tab[w.e * BS + w.c];
+        cdf[i] = (uint16_t)tab[w.e * TableStride<BS>::k32 + w.c];
     }
 }
 
-// Load the block's tables into LDS as tab[entry * BS + lane] (32-bit words).
+// Load the block's tables into LDS as tab[entry * stride + lane] (32-bit words).
 template <int BS>
 __device__ __forceinline__ void stage_tables(uint32_t *tab, const uint16_t *cdf, int lp, int64_t ch0, int64_t nc)
 {
@@ -78,11 +89,11 @@ __device__ __forceinline__ void stage_tables(uint32_t *tab, const uint16_t *cdf,
     const int total = (int)nvalid * lp;
     TableWalk w(threadIdx.x, BS, lp);
     for (int i = threadIdx.x; i < total; i += BS, w.next(lp)) {
-        tab[w.e * BS + w.c] = cdf[i];
+        tab[w.e * TableStride<BS>::k32 + w.c] = cdf[i];
     }
 }
 
-// The stream kernels keep their tables in LDS as 16-bit entries tab[entry * BS + lane]
+// The stream kernels keep their tables in LDS as 16-bit entries tab[entry * stride + lane]
 // (half the footprint, twice the resident waves).  The end of a table, 2^16, does not fit
 // and is substituted where the last symbol's upper bound is read.
 template <int BS>
@@ -92,7 +103,7 @@ __device__ __forceinline__ void stage_tables16(uint16_t *tab, const uint16_t *cd
     const int total = (int)nvalid * lp;
     TableWalk w(threadIdx.x, BS, lp);
     for (int i = threadIdx.x; i < total; i += BS, w.next(lp)) {
-        tab[w.e * BS + w.c] = cdf[i];
+        tab[w.e * TableStride<BS>::k16 + w.c] = cdf[i];
     }
 }
 
@@ -103,7 +114,7 @@ __device__ __forceinline__ void write_tables16(const uint16_t *tab, uint16_t *cd
     const int total = (int)nvalid * lp;
     TableWalk w(threadIdx.x, BS, lp);
     for (int i = threadIdx.x; i < total; i += BS, w.next(lp)) {
-        cdf[i] = tab[w.e * BS + w.c];
+        cdf[i] = tab[w.e * TableStride<BS>::k16 + w.c];
     }
 }
 
@@ -113,24 +124,25 @@ __device__ __forceinline__ void write_tables16(const uint16_t *tab, uint16_t *cd
 template <int BS>
 __device__ __forceinline__ void normalize_column16(uint16_t *col, int lp, int max_bins, uint32_t total)
 {
+    constexpr int kS = TableStride<BS>::k16;
     const uint32_t scale = 0xFFFFu - (uint32_t)max_bins;
     uint32_t running = 0;
     if ((total & (total - 1)) == 0) {
         const int sh = 31 - __builtin_clz(total);
         for (int i = 0; i < lp; ++i) {
-            running += col[i * BS];
-            col[i * BS] = (uint16_t)(((scale * running) >> sh) + (uint32_t)i);
+            running += col[i * kS];
+            col[i * kS] = (uint16_t)(((scale * running) >> sh) + (uint32_t)i);
         }
     } else {
         const float inv = __fdiv_rn(1.0f, (float)total);
         for (int i = 0; i < lp; ++i) {
-            running += col[i * BS];
+            running += col[i * kS];
             const uint32_t x = scale * running;                  // < 2^32, quotient < 2^16
             uint32_t q = (uint32_t)((float)x * inv);
             int32_t rem = (int32_t)(x - q * total);
             if (rem < 0) { q--; rem += (int32_t)total; }
             if (rem >= (int32_t)total) q++;
-            col[i * BS] = (uint16_t)(q + (uint32_t)i);
+            col[i * kS] = (uint16_t)(q + (uint32_t)i);
         }
     }
 }
@@ -161,13 +173,14 @@ __global__ __launch_bounds__(BS) void calculate_cdf_kernel(CdfArgs a)
     const int64_t ch = (int64_t)ctile * BS + tid;
     // byte symbols: one 32-bit counter per (entry, lane); packed symbols (the fused path, whose
     // symbols all lie inside the table): 16-bit counters, two lanes to a word, as in the encoder
+    constexpr int kS16 = TableStride<BS>::k16, kS32 = TableStride<BS>::k32;
     uint32_t *col = smem + tid;
     uint16_t *tab16 = reinterpret_cast<uint16_t *>(smem);
     if (PACKED) {
-        for (int i = 0; i < lp; ++i) tab16[i * BS + tid] = 0;
+        for (int i = 0; i < lp; ++i) tab16[i * kS16 + tid] = 0;
         __syncthreads();                     // a lane's neighbour shares its words
     } else {
-        for (int i = 0; i < lp; ++i) col[i * BS] = 0;
+        for (int i = 0; i < lp; ++i) col[i * kS32] = 0;
     }
 
     const int64_t t0 = chunk * a.g.S;
@@ -184,11 +197,11 @@ __global__ __launch_bounds__(BS) void calculate_cdf_kernel(CdfArgs a)
                 for (int j = 0; j < 8; ++j) v[j] = p[(t + j) * a.s1];
 #pragma unroll
                 for (int j = 0; j < 8; ++j)
-                    if (v[j] < mb) atomicAdd(col + (v[j] + 1) * BS, 1u);      // no value returned: one LDS operation
+                    if (v[j] < mb) atomicAdd(col + (v[j] + 1) * kS32, 1u);      // no value returned: one LDS operation
             }
             for (; t < t1; ++t) {
                 const uint32_t v = p[t * a.s1];
-                if (v < mb) atomicAdd(col + (v + 1) * BS, 1u);
+                if (v < mb) atomicAdd(col + (v + 1) * kS32, 1u);
             }
         } else {
             uint32_t *const pair = smem + (tid >> 1);
@@ -209,7 +222,7 @@ __global__ __launch_bounds__(BS) void calculate_cdf_kernel(CdfArgs a)
                     for (int j = 0; j < 4 * kBatch; ++j) {
                         uint32_t s = (v[j >> 2] >> (8 * (j & 3))) & 0xFFu;
                         s = s < mb - 1u ? s : mb - 1u;
-                        if (w0 * 4 + j < n) atomicAdd(pair + (s + 1) * (BS / 2), one);
+                        if (w0 * 4 + j < n) atomicAdd(pair + (s + 1) * (kS16 / 2), one);
                     }
                 }
             }

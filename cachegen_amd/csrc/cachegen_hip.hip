@@ -312,6 +312,11 @@ int cg_decode_kv(const int16_t *cdf, int max_bins, const void *maxima, int max_d
     if (delta_group < 0 || delta_group > kSub) return fail(CG_ERR_ARG, "decode_kv: delta_group must be in [0, %d]", kSub);
     const int64_t C = H * D, rows = 2 * L;
     if (D > INT_MAX) return fail(CG_ERR_ARG, "decode_kv: head size too large");
+    // the kernel stores through a buffer descriptor per block: a channel's byte offset plus a
+    // token row's byte offset inside one stream's token range must fit 32 bits
+    if (ot < 0 || oh < 0 || ((H - 1) * oh + (D - 1) + (int64_t)(kSub - 1) * ot) * 2 + 2 > 0xFFFFFFFFll)
+        return fail(CG_ERR_ARG, "decode_kv: negative output strides, or %d token rows of one layer's keys or values "
+                                "span 4 GiB or more", kSub);
     const int64_t nsub = cg_num_subchunks(T, chunk_tokens);
     const int block = pick_block(C, max_bins + 1);
     DecodeArgs a;

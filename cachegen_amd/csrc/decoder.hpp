@@ -29,20 +29,27 @@ namespace {
 // Bits past the end of a stream are whatever follows it in memory instead of the reference's
 // zeros (dec_new.cu:223-233): the coder's two closing bits place the code value inside
 // the final interval for every continuation, so the n symbols that were encoded decode
-// identically.  Word loads are clamped to the last word of the byte buffer.
+// identically.  Word loads past the last word of the byte buffer return zeros.
+
+// Fourth word of a buffer descriptor for raw (untyped, unswizzled) access on gfx9-family
+// GPUs: 32-bit data format, everything else off.
+constexpr int kBufferWord3 = 0x00020000;
+
 struct BitReader {
-    const uint8_t *base;     // the aligned word holding the stream's first byte
-    uint32_t last;           // byte offset from `base` of the last word that may be read
-    uint32_t pos;            // byte offset from `base` of the next word to fetch
+    // Words are fetched with buffer loads: the descriptor (uniform over the wavefront) covers
+    // the byte buffer from the wavefront's first stream to its last readable word, a lane
+    // addresses it with a 32-bit offset, and a load outside it returns zero instead of faulting.
+    __amdgpu_buffer_rsrc_t rsrc;
+    uint32_t pos;            // byte offset inside the descriptor's range of the next word to fetch
     uint64_t win;            // the next `avail` bits of the stream, left-aligned, zeros below
     int avail;
     uint32_t nextw;          // the word after the window, as loaded
 
     __device__ __forceinline__ uint32_t raw()
     {
-        const uint32_t at = pos < last ? pos : last;
+        const uint32_t w = __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)pos, 0, 0);
         pos += 4;
-        return *reinterpret_cast<const uint32_t *>(base + at);
+        return w;
     }
 
     // position on the stream that begins `begin` bytes after the 4-byte aligned `window`,
@@ -54,10 +61,16 @@ struct BitReader {
         begin = begin < 0 ? 0 : (begin > last_word + 3 ? last_word + 3 : begin);     // last_word is a word's first byte
         const uint32_t skip = (uint32_t)begin & 3u;
         const int64_t first_word = begin - skip;
-        base = window + first_word;
-        const int64_t room = last_word - first_word;
-        last = room < 0 ? 0u : (room > 0xFFFFFFF0ll ? 0xFFFFFFF0u : (uint32_t)room);
-        pos = 0;
+        // the descriptor starts at the first word of the wavefront's first active lane; a lane
+        // whose stream lies before it or 4 GiB behind it gets an offset that wraps, which
+        // reads zeros or some other place inside the buffer
+        const uint32_t org_lo = __builtin_amdgcn_readfirstlane((uint32_t)first_word);
+        const uint32_t org_hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)first_word >> 32));
+        const int64_t origin = (int64_t)(((uint64_t)org_hi << 32) | org_lo);
+        const int64_t room = last_word + 4 - origin;                           // >= 4
+        rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(window + origin), 0,
+                                                 (int)(room > 0xFFFFFFFFll ? 0xFFFFFFFFu : (uint32_t)room), kBufferWord3);
+        pos = (uint32_t)(first_word - origin);
         const uint32_t b0 = __builtin_bswap32(raw()), b1 = __builtin_bswap32(raw());
         const uint32_t b2 = __builtin_bswap32(raw());
         nextw = raw();
@@ -72,7 +85,9 @@ struct BitReader {
     // off = (off << n) | next n bits, 0 <= n <= 31 and n <= avail
     __device__ __forceinline__ uint32_t shift_in(uint32_t off, int n)
     {
-        off = (off << n) | __builtin_amdgcn_ubfe((uint32_t)(win >> 32), (uint32_t)(32 - n), (uint32_t)n);   // n = 0 extracts nothing
+        // two 64-bit shifts: {off, top word of the window} and the window itself
+        const uint64_t pair = (((uint64_t)off << 32) | (uint32_t)(win >> 32)) << n;
+        off = (uint32_t)(pair >> 32);
         win <<= n;
         avail -= n;
         return off;
@@ -82,7 +97,8 @@ struct BitReader {
     __device__ __forceinline__ void top_up()
     {
         if (avail <= 32) {                      // the low word is empty
-            win |= (((uint64_t)__builtin_bswap32(nextw)) << 32) >> (avail & 63);
+            const uint64_t in = (((uint64_t)__builtin_bswap32(nextw)) << 32) >> (avail & 63);
+            win = (((win >> 32) | (in >> 32)) << 32) | (uint32_t)in;
             avail += 32;
             nextw = raw();
         }
@@ -150,7 +166,11 @@ struct DecodeLane {
     // of two for the second), read once per stream: two LDS round trips less per symbol
     uint32_t probe1, probe2_lo, probe2_hi;
     uint8_t *osym;
-    uint16_t *okv;
+    // dequantised output: one buffer descriptor per block, starting at the block's first token
+    // row of its (layer, K/V) slab; a lane adds its channel's byte offset, a token row is
+    // reached through the scalar offset
+    __amdgpu_buffer_rsrc_t orsrc;
+    uint32_t ovoff;
     float anchor;              // reconstructed anchor row value (delta mode)
     int phase;                 // position of the token inside its group (delta mode)
 };
@@ -173,19 +193,7 @@ __device__ __forceinline__ void decode_symbol(const DecodeArgs &a, DecodeLane &s
     float q = 0.0f;                    // (symbol - C) / C
     const bool full_range = s.span == 0;
     const uint32_t sh = s.span >> 16, sl = s.span & 0xFFFFu;
-    if (LOG2 >= 2 && __builtin_expect(full_range, 0)) {
-        // full range (a stream's first symbol, hardly ever later): T(m) = cdf[m] << 16, so
-        // table values are compared with off >> 16
-        const uint32_t key = s.off >> 16;
-#pragma unroll
-        for (int step = kStep1; step >= 1; step >>= 1)
-            p = (lds_entry(p, step * kRow) <= key) ? p + step * kRow : p;
-        const uint32_t c_lo = lds_entry(p, 0);
-        const uint32_t c_hi = (SAFE && p == plast) ? 0x10000u : lds_entry(p, kRow);
-        if (OUT != OUT_SYMBOLS) q = *(lds_f32 *)(p + s.lutoff);
-        t_lo = c_lo << 16;
-        width = (c_hi - c_lo) << 16;
-    } else if (LOG2 >= 2) {
+    if (LOG2 >= 2) {
         // largest m with T(m) <= off, probed with the lower bound sh * c <= T(c), which can
         // only overshoot; the first two probes compare entries held in registers
         const bool up1 = mul24(sh, s.probe1) <= s.off;
@@ -202,17 +210,35 @@ __device__ __forceinline__ void decode_symbol(const DecodeArgs &a, DecodeLane &s
         uint32_t c_lo = lds_entry(p, 0);
         uint32_t c_hi = lds_entry(p, kRow);
         if (OUT != OUT_SYMBOLS) q = *(lds_f32 *)(p + s.lutoff);
-        t_lo = scale_span(sh, sl, c_lo);
-        // entry 0 is 0 (forced when the tables are staged), so this stops there at the latest
-        while (__builtin_expect(t_lo > s.off, 0)) {
-            p -= kRow;
-            c_hi = c_lo;
-            c_lo = lds_entry(p, 0);
-            if (OUT != OUT_SYMBOLS) q = *(lds_f32 *)(p + s.lutoff);
-            t_lo = scale_span(sh, sl, c_lo);
-        }
         if (SAFE && p == plast) c_hi = 0x10000u;                                // dec_new.cu:278
+        t_lo = scale_span(sh, sl, c_lo);
         width = scale_span(sh, sl, c_hi) - t_lo;
+        // One test for what is left: off - t_lo wraps when the search overshot, and the full
+        // range (span 0 modulo 2^32: a stream's first symbol, hardly ever later) gives width 0.
+        if (__builtin_expect(s.off - t_lo >= width, 0)) {
+            if (full_range) {
+                // T(m) = cdf[m] << 16, so table values are compared with off >> 16
+                const uint32_t key = s.off >> 16;
+                p = s.colp;
+#pragma unroll
+                for (int step = kStep1; step >= 1; step >>= 1)
+                    p = (lds_entry(p, step * kRow) <= key) ? p + step * kRow : p;
+                c_lo = lds_entry(p, 0);
+                c_hi = (SAFE && p == plast) ? 0x10000u : lds_entry(p, kRow);
+                t_lo = c_lo << 16;
+                width = (c_hi - c_lo) << 16;
+            } else {
+                // entry 0 is 0 (forced when the tables are staged), so this stops there at the latest
+                while (t_lo > s.off) {
+                    p -= kRow;
+                    c_hi = c_lo;
+                    c_lo = lds_entry(p, 0);
+                    t_lo = scale_span(sh, sl, c_lo);
+                }
+                width = scale_span(sh, sl, c_hi) - t_lo;
+            }
+            if (OUT != OUT_SYMBOLS) q = *(lds_f32 *)(p + s.lutoff);
+        }
     } else {
         int lo_i = 0, hi_i = lp - 1;
         for (int step = 0; step < nsteps; ++step) {
@@ -250,8 +276,7 @@ __device__ __forceinline__ void decode_symbol(const DecodeArgs &a, DecodeLane &s
         uint32_t bits;
         if (OUT == OUT_BF16) bits = SAFE ? float_to_bf16_bits(v) : float_to_bf16_bits_no_nan(v);
         else bits = float_to_f16_bits(v);
-        *s.okv = (uint16_t)bits;
-        s.okv += a.ot;
+        __builtin_amdgcn_raw_buffer_store_b16((short)bits, s.orsrc, (int)s.ovoff, (int)((uint32_t)i * (uint32_t)a.ot * 2u), 0);
     }
     if (last_symbol) return;                    // no update after the last symbol
     s.low += t_lo;
@@ -263,7 +288,10 @@ __device__ __forceinline__ void decode_symbol(const DecodeArgs &a, DecodeLane &s
     // inside the word because the interval is wider than one
     const uint32_t z = ((s.low & high) | (~s.low & 0xFFFFFFFFu)) << ((n1 + 1) & 31);   // one bit-field insert
     const int n = n1 + __builtin_clz(z);
-    s.low = (s.low << n) & 0x7FFFFFFFu;
+    // bit 31 of low would be cleared here (the underflow steps subtract a quarter); it is left
+    // as it falls: low and high = low + width - 1 then carry the same extra 2^31 modulo 2^32,
+    // and only low ^ high and bits below the first differing one are looked at
+    s.low <<= n;
     s.span = width << n;
     s.off = s.rd.shift_in(s.off, n);
 }
@@ -357,14 +385,19 @@ __global__ __launch_bounds__(BS) void decode_streams_kernel(DecodeArgs a)
     s.colp = (lds_char *)(rows + 2 * tid);
     s.lutoff = DecodeLayout<BS, OUT>::kQuot - 2 * tid;
     s.osym = nullptr;
-    s.okv = nullptr;
+    s.ovoff = 0;
     s.anchor = 0.0f;
     s.phase = 0;
     if (OUT == OUT_SYMBOLS) {
         s.osym = a.out_sym + id.row * a.o0 + id.t0 * a.o1 + id.ch * a.o2;
     } else {
         const int64_t h = id.ch / a.D;
-        s.okv = a.out_kv + l * a.ol + kvi * a.okv + id.t0 * a.ot + h * a.oh + (id.ch - h * a.D);
+        const int64_t first_row = l * a.ol + kvi * a.okv + id.t0 * a.ot;             // uniform over the block
+        const uint32_t fr_lo = __builtin_amdgcn_readfirstlane((uint32_t)first_row);
+        const uint32_t fr_hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)first_row >> 32));
+        s.orsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(a.out_kv + (int64_t)(((uint64_t)fr_hi << 32) | fr_lo)), 0,
+                                                    (int)0xFFFFFFFFu, kBufferWord3);
+        s.ovoff = (uint32_t)((h * a.oh + (id.ch - h * a.D)) * 2);                    // the host checks that this fits
     }
     lds_f32 *rmp = (lds_f32 *)rowmax;
 

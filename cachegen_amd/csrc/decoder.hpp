@@ -149,6 +149,18 @@ __device__ __forceinline__ uint32_t lds_entry(lds_char *p, int byte_offset)
     return *(lds_u16 *)(p + byte_offset);
 }
 
+// Entries at p and p + ROW bytes into the upper halves of `lo` and `hi` (entry << 16), whose
+// lower halves must be zero on entry and are zero on return: the hardware either keeps them
+// or clears them.  The compiler does not count loads issued from inline assembly, so the wait
+// for them is part of it.
+template <int ROW>
+__device__ __forceinline__ void lds_entries_high(lds_char *p, uint32_t &lo, uint32_t &hi)
+{
+    asm volatile("ds_read_u16_d16_hi %0, %2\n\tds_read_u16_d16_hi %1, %2 offset:%3\n\ts_waitcnt lgkmcnt(0)"
+                 : "+v"(lo), "+v"(hi)
+                 : "v"(p), "n"(ROW));
+}
+
 // float32 -> bfloat16 bits, round to nearest even, for anything but a NaN
 __device__ __forceinline__ uint32_t float_to_bf16_bits_no_nan(float f)
 {
@@ -165,6 +177,9 @@ struct DecodeLane {
     // the entries the first two probes of the unrolled search look at (one for the first, one
     // of two for the second), read once per stream: two LDS round trips less per symbol
     uint32_t probe1, probe2_lo, probe2_hi;
+    // the decoded symbol's two table entries, each shifted left by 16: only ever written by
+    // loads into the upper half, so that the lower halves stay zero
+    uint32_t bound_lo, bound_hi;
     uint8_t *osym;
     // dequantised output: one buffer descriptor per block, starting at the block's first token
     // row of its (layer, K/V) slab; a lane adds its channel's byte offset, a token row is
@@ -189,7 +204,7 @@ __device__ __forceinline__ void decode_symbol(const DecodeArgs &a, DecodeLane &s
     constexpr int kStep1 = first_probe(LOG2, SKIP), kStep2 = kStep1 >> 1;
     lds_char *p = s.colp;              // entry of the decoded symbol
     lds_char *const plast = s.colp + (lp - 2) * kRow;
-    uint32_t t_lo, width;
+    uint32_t t_lo, width, rel;         // rel = off - t_lo
     float q = 0.0f;                    // (symbol - C) / C
     const bool full_range = s.span == 0;
     const uint32_t sh = s.span >> 16, sl = s.span & 0xFFFFu;
@@ -207,15 +222,16 @@ __device__ __forceinline__ void decode_symbol(const DecodeArgs &a, DecodeLane &s
             p = (mul24(sh, lds_entry(p, step * kRow)) <= s.off) ? p + step * kRow : p;
         // both bounds and the quotient in one round trip (entry lp - 1 exists, so the upper
         // bound of the last symbol can be read and then replaced)
-        uint32_t c_lo = lds_entry(p, 0);
-        uint32_t c_hi = lds_entry(p, kRow);
         if (OUT != OUT_SYMBOLS) q = *(lds_f32 *)(p + s.lutoff);
-        if (SAFE && p == plast) c_hi = 0x10000u;                                // dec_new.cu:278
-        t_lo = scale_span(sh, sl, c_lo);
-        width = scale_span(sh, sl, c_hi) - t_lo;
+        lds_entries_high<kRow>(p, s.bound_lo, s.bound_hi);
+        // T(c) = (span * c) >> 16 = high word of span * (c << 16) for c < 2^16; the one entry
+        // that is 2^16, the upper bound of the last symbol (dec_new.cu:278), gives the span
+        t_lo = __umulhi(s.span, s.bound_lo);
+        width = ((SAFE && p == plast) ? s.span : __umulhi(s.span, s.bound_hi)) - t_lo;
         // One test for what is left: off - t_lo wraps when the search overshot, and the full
         // range (span 0 modulo 2^32: a stream's first symbol, hardly ever later) gives width 0.
-        if (__builtin_expect(s.off - t_lo >= width, 0)) {
+        rel = s.off - t_lo;
+        if (__builtin_expect(rel >= width, 0)) {
             if (full_range) {
                 // T(m) = cdf[m] << 16, so table values are compared with off >> 16
                 const uint32_t key = s.off >> 16;
@@ -223,21 +239,25 @@ __device__ __forceinline__ void decode_symbol(const DecodeArgs &a, DecodeLane &s
 #pragma unroll
                 for (int step = kStep1; step >= 1; step >>= 1)
                     p = (lds_entry(p, step * kRow) <= key) ? p + step * kRow : p;
-                c_lo = lds_entry(p, 0);
-                c_hi = (SAFE && p == plast) ? 0x10000u : lds_entry(p, kRow);
+                const uint32_t c_lo = lds_entry(p, 0);
+                const uint32_t c_hi = (SAFE && p == plast) ? 0x10000u : lds_entry(p, kRow);
                 t_lo = c_lo << 16;
                 width = (c_hi - c_lo) << 16;
             } else {
                 // entry 0 is 0 (forced when the tables are staged), so this stops there at the latest
+                bool top = SAFE && p == plast;
+                uint32_t b_lo = s.bound_lo, b_hi = s.bound_hi;
                 while (t_lo > s.off) {
                     p -= kRow;
-                    c_hi = c_lo;
-                    c_lo = lds_entry(p, 0);
-                    t_lo = scale_span(sh, sl, c_lo);
+                    b_hi = b_lo;
+                    top = false;
+                    b_lo = lds_entry(p, 0) << 16;
+                    t_lo = __umulhi(s.span, b_lo);
                 }
-                width = scale_span(sh, sl, c_hi) - t_lo;
+                width = (top ? s.span : __umulhi(s.span, b_hi)) - t_lo;
             }
             if (OUT != OUT_SYMBOLS) q = *(lds_f32 *)(p + s.lutoff);
+            rel = s.off - t_lo;
         }
     } else {
         int lo_i = 0, hi_i = lp - 1;
@@ -259,6 +279,7 @@ __device__ __forceinline__ void decode_symbol(const DecodeArgs &a, DecodeLane &s
             t_lo = scale_span(sh, sl, c_lo);
             width = scale_span(sh, sl, c_hi) - t_lo;
         }
+        rel = s.off - t_lo;
     }
     if (OUT == OUT_SYMBOLS) {
         s.osym[(int64_t)i * a.o1] = (uint8_t)((uint32_t)(p - s.colp) / (uint32_t)kRow);
@@ -280,7 +301,7 @@ __device__ __forceinline__ void decode_symbol(const DecodeArgs &a, DecodeLane &s
     }
     if (last_symbol) return;                    // no update after the last symbol
     s.low += t_lo;
-    s.off -= t_lo;
+    s.off = rel;
     const uint32_t high = s.low + width - 1u;
     const int n1 = __builtin_clz(s.low ^ high);
     // E3 run: positions below the first differing bit where low has 1 and high has 0, i.e.
@@ -308,6 +329,8 @@ __device__ __forceinline__ void decode_lane(const DecodeArgs &a, DecodeLane &s, 
         s.probe1 = lds_entry(s.colp, kStep1 * kRow);
         s.probe2_lo = lds_entry(s.colp, kStep2 * kRow);
         s.probe2_hi = lds_entry(s.colp, (kStep1 + kStep2) * kRow);
+        s.bound_lo = 0;
+        s.bound_hi = 0;
     }
     for (int i0 = 0; i0 < n; i0 += 4, rmp += 4) {
         // the maxima of the next four token rows (the array is padded to a multiple of four)

@@ -110,4 +110,21 @@ __device__ __forceinline__ uint32_t scale_span(uint32_t sh, uint32_t sl, uint32_
     return mul24(sh, c) + (mul24(sl, c) >> 16);
 }
 
+// Pointers into LDS, for loads with immediate offsets.
+typedef __attribute__((address_space(3))) const uint16_t lds_u16;
+typedef __attribute__((address_space(3))) const float lds_f32;
+typedef __attribute__((address_space(3))) const char lds_char;
+
+// Entries at p and p + ROW bytes into the upper halves of `lo` and `hi` (entry << 16), whose
+// lower halves must be zero on entry and are zero on return: the hardware either keeps them
+// or clears them.  The compiler does not count loads issued from inline assembly, so the wait
+// for them is part of it.
+template <int ROW>
+__device__ __forceinline__ void lds_entries_high(lds_char *p, uint32_t &lo, uint32_t &hi)
+{
+    asm volatile("ds_read_u16_d16_hi %0, %2\n\tds_read_u16_d16_hi %1, %2 offset:%3\n\ts_waitcnt lgkmcnt(0)"
+                 : "+v"(lo), "+v"(hi)
+                 : "v"(p), "n"(ROW));
+}
+
 }  // namespace

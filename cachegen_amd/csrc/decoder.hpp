@@ -140,25 +140,10 @@ struct DecodeLayout {
     static constexpr int kQuot = 2 * BS;          // byte offset of the quotient inside a row
 };
 
-typedef __attribute__((address_space(3))) const uint16_t lds_u16;
-typedef __attribute__((address_space(3))) const float lds_f32;
-typedef __attribute__((address_space(3))) const char lds_char;
 
 __device__ __forceinline__ uint32_t lds_entry(lds_char *p, int byte_offset)
 {
     return *(lds_u16 *)(p + byte_offset);
-}
-
-// Entries at p and p + ROW bytes into the upper halves of `lo` and `hi` (entry << 16), whose
-// lower halves must be zero on entry and are zero on return: the hardware either keeps them
-// or clears them.  The compiler does not count loads issued from inline assembly, so the wait
-// for them is part of it.
-template <int ROW>
-__device__ __forceinline__ void lds_entries_high(lds_char *p, uint32_t &lo, uint32_t &hi)
-{
-    asm volatile("ds_read_u16_d16_hi %0, %2\n\tds_read_u16_d16_hi %1, %2 offset:%3\n\ts_waitcnt lgkmcnt(0)"
-                 : "+v"(lo), "+v"(hi)
-                 : "v"(p), "n"(ROW));
 }
 
 // float32 -> bfloat16 bits, round to nearest even, for anything but a NaN
@@ -343,7 +328,7 @@ __device__ __forceinline__ void decode_lane(const DecodeArgs &a, DecodeLane &s, 
         for (int j = 0; j < 4; ++j) {
             const int i = i0 + j;
             if (i >= n) break;
-            if ((j & 1) == 0) s.rd.top_up();
+            if (j == 0) s.rd.top_up();
             else if (__builtin_expect(s.rd.avail < 18, 0)) s.rd.top_up();
             decode_symbol<BS, LOG2, OUT, SKIP, SAFE>(a, s, lp, nsteps, rm[j], i, i == n - 1);
         }

@@ -116,14 +116,19 @@ struct BitWriter {
 // span to span << n for E1/E2 and E3 steps alike.
 template <int BS, bool ALIGNED>
 struct RangeEncoder {
-    const uint16_t *col;    // this lane's table column: entry e at col[e * TableStride<BS>::k16]
+    lds_char *col;          // this lane's table column: entry e at byte e * 2 * TableStride<BS>::k16
     uint32_t smax;          // lp - 2: the largest symbol
     uint32_t low, span, pend;
+    // the coded symbol's two table entries, each shifted left by 16: only ever written by
+    // loads into the upper half, so that the lower halves stay zero
+    uint32_t bound_lo, bound_hi;
     BitWriter<ALIGNED> w;
 
     __device__ __forceinline__ void init(const uint16_t *column, int lp, uint8_t *dst, int wstride, int cap)
     {
-        col = column;
+        col = (lds_char *)column;
+        bound_lo = 0;
+        bound_hi = 0;
         smax = (uint32_t)(lp - 2);
         low = 0;
         span = 0;
@@ -143,18 +148,19 @@ struct RangeEncoder {
     __device__ __forceinline__ void put_symbol(uint32_t s)
     {
         s = s < smax ? s : smax;                        // keep table reads inside the table
-        constexpr int kS = TableStride<BS>::k16;
-        const uint32_t c_lo = col[s * kS];
-        const uint32_t c_next = col[s * kS + kS];
-        const uint32_t c_hi = (SENTINEL && s == smax) ? 0x10000u : c_next;
+        constexpr int kRow = 2 * TableStride<BS>::k16;
+        lds_entries_high<kRow>(col + s * kRow, bound_lo, bound_hi);
+        // the upper bound of symbol smax is 2^16 and not the table's last entry; shifted left
+        // by 16 that is 0 modulo 2^32, and T(2^16) is the span
+        const bool top = SENTINEL && s == smax;
         uint32_t t_lo, width;
         if (__builtin_expect(span == 0, 0)) {
-            t_lo = c_lo << 16;
-            width = (c_hi - c_lo) << 16;
+            t_lo = bound_lo;                                // c << 16
+            width = (top ? 0u : bound_hi) - bound_lo;
         } else {
-            const uint32_t sh = span >> 16, sl = span & 0xFFFFu;
-            t_lo = scale_span(sh, sl, c_lo);
-            width = scale_span(sh, sl, c_hi) - t_lo;
+            // T(c) = (span * c) >> 16 = high word of span * (c << 16)
+            t_lo = __umulhi(span, bound_lo);
+            width = (top ? span : __umulhi(span, bound_hi)) - t_lo;
         }
         low += t_lo;
         const uint32_t high = low + width - 1u;

@@ -22,10 +22,11 @@ namespace {
 //
 // The stream is read through aligned big-endian words into a 64-bit window of unread bits.
 // Every lane of a wavefront runs the refill code whenever one lane needs it, so the window
-// is topped up at fixed points, once per two symbols, instead of whenever a lane runs dry:
-// after a top-up it holds more than 32 bits, a symbol of a table without zero-width entries
-// consumes at most 18 (the span stays above 2^30), and the one case left (fewer than 18 bits
-// before the second symbol of a pair) takes an extra top-up.
+// is topped up at fixed points, once per four symbols, instead of whenever a lane runs dry:
+// after a top-up it holds more than 32 bits, which streams of a few bits per symbol do not
+// use up in four symbols; a symbol of a table without zero-width entries consumes at most 18
+// (the span stays above 2^30), so the case left (fewer than 18 bits before one of the other
+// three symbols) takes an extra top-up.
 // Bits past the end of a stream are whatever follows it in memory instead of the reference's
 // zeros (dec_new.cu:223-233): the coder's two closing bits place the code value inside
 // the final interval for every continuation, so the n symbols that were encoded decode

@@ -14,9 +14,9 @@ namespace {
 // ---- encoder (enc_new.cu:21-97, 253-307) -------------------------------------------
 // Bits are collected MSB-first in a 64-bit accumulator and leave as big-endian 32-bit words.
 // Every lane of a wavefront runs the store code whenever one lane has a word ready, so words
-// are written at fixed points, once per two symbols, instead of whenever a lane's
-// accumulator fills; the accumulator takes the two symbols in between (a put that would not
-// fit writes a word first).
+// are written at fixed points, once per four symbols (per two, for byte symbols), instead of
+// whenever a lane's accumulator fills; the accumulator takes the symbols in between (a put
+// that would not fit writes a word first).
 // The E1/E2 run of a symbol is emitted at once: the n1 = clz(low ^ high) leading bits
 // agree, and the pending complements go in after the first of them, which in arithmetic
 // is  bits + ((2^pend - 1) << (n1 - 1))  over n1 + pend bits.  The E3 run k is the number
@@ -143,7 +143,7 @@ struct RangeEncoder {
 
     // SENTINEL: symbol smax may occur, whose upper bound is 2^16 and not the table's last
     // entry (enc_new.cu:270)
-    // FIRST: the symbol directly follows a flush_word (the first of a pair)
+    // FIRST: the symbol directly follows a flush_word (the first of a group)
     template <bool SENTINEL, bool FIRST>
     __device__ __forceinline__ void put_symbol(uint32_t s)
     {
@@ -313,8 +313,7 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
                     const int t = (h * 32 + w) * 4;            // first token of the word
                     if (t + 0 < id.n) enc.template put_symbol<SENTINEL, true>(v & 0xFFu);
                     if (t + 1 < id.n) enc.template put_symbol<SENTINEL, false>((v >> 8) & 0xFFu);
-                    enc.w.flush_word();
-                    if (t + 2 < id.n) enc.template put_symbol<SENTINEL, true>((v >> 16) & 0xFFu);
+                    if (t + 2 < id.n) enc.template put_symbol<SENTINEL, false>((v >> 16) & 0xFFu);
                     if (t + 3 < id.n) enc.template put_symbol<SENTINEL, false>(v >> 24);
                     enc.w.flush_word();
                 }

@@ -175,7 +175,9 @@ struct RangeEncoder {
             w.put(bits & ((1u << (n1 - 1)) - 1u), n1 - 1);
         } else {
             const uint32_t bits = __builtin_amdgcn_ubfe(low, (uint32_t)(32 - n1), (uint32_t)n1);
-            const uint32_t fill = ((1u << (pe & 31)) - 1u) << ((n1 - 1) & 31);
+            // ((1 << pe) - 1) << (n1 - 1), pe <= 31 here; with n1 = 0, pe is 0 and so is the mask
+            uint32_t fill;
+            asm("v_bfm_b32 %0, %1, %2" : "=v"(fill) : "v"(pe), "v"(n1 - 1));
             w.template put<FIRST>(bits + fill, m);
         }
         // E3 run: leading zeros of (~low | high) below the first differing bit

@@ -161,7 +161,11 @@ int cg_scan_lengths(const int32_t *lengths, int64_t n, int64_t *offsets,
  * cdf, maxima, offsets, payload: as written by cg_encode_kv (maxima in max_dt);
  *             whole aligned 32-bit words of the payload are loaded, see
  *             cg_decode_fast_prefsum
- * out         device fp16/bf16 KV cache (out_dt, strides (ol, okv, ot, oh, 1)), written */
+ * out         device fp16/bf16 KV cache (out_dt, strides (ol, okv, ot, oh, 1)), written.
+ *             ot and oh must not be negative, and 256 token rows of one layer's keys or
+ *             values must span less than 4 GiB (((H-1)*oh + D-1 + 255*ot) * 2 + 2 bytes):
+ *             the kernel addresses them with a 32-bit offset from a per-block base;
+ *             CG_ERR_ARG otherwise */
 int cg_decode_kv(const int16_t *cdf, int max_bins, const void *maxima, int max_dt,
                  const int64_t *offsets, const uint8_t *payload, int64_t payload_bytes,
                  const float *key_bins, const float *value_bins,

@@ -33,6 +33,24 @@ def test_chunk_arithmetic():
     assert lib.cg_encode_kv_workspace(2, 512, 512, 512) >= 2 * 2 * 512 * 512 + 2 * 4 * 512 * 256
 
 
+def test_decode_kv_refuses_output_strides_it_cannot_address():
+    """Argument checks only: they come before anything touches a device, so the pointers here
+    are never dereferenced."""
+    from cachegen_amd import _lib
+    lib = _lib.lib()
+    fake = 4096
+    L, T, H, D = 2, 256, 8, 128
+
+    def call(ot, oh):
+        return lib.cg_decode_kv(fake, 32, fake, 0, fake, fake, 1024, fake, fake, L, T, H, D, 256, 0,
+                                fake, 0, 2 * T * H * D, T * H * D, ot, oh, None)
+
+    assert call(-H * D, D) != 0 and b"strides" in lib.cg_last_error()
+    assert call(H * D, -D) != 0
+    assert call(1 << 24, D) != 0 and b"4 GiB" in lib.cg_last_error()         # 255 rows of 32 MiB
+    assert call(D, 1 << 29) != 0                                           # heads 1 GiB apart
+
+
 def test_bins_tables_match_reference_tables(monkeypatch):
     from cachegen_amd.serde.cachegen_basics import CacheGenConfig, make_key_bins, make_value_bins
     cfg = CacheGenConfig.from_model_name("lmsys/longchat-7b-16k")

@@ -55,18 +55,22 @@ struct BitReader {
 
     // position on the stream that begins `begin` bytes after the 4-byte aligned `window`,
     // whose last readable word is at byte offset `last_word`; returns the first 32 bits
-    __device__ __forceinline__ uint32_t start(const uint8_t *window, int64_t last_word, int64_t begin)
+    // `lowest`: the smallest `begin` among the wavefront's lanes, the same value in every lane
+    __device__ __forceinline__ uint32_t start(const uint8_t *window, int64_t last_word, int64_t begin, int64_t lowest)
     {
         // a start outside the buffer (offsets that are not running sums of stream lengths) is
         // moved inside it: such a stream decodes to garbage, never to a read out of bounds
-        begin = begin < 0 ? 0 : (begin > last_word + 3 ? last_word + 3 : begin);     // last_word is a word's first byte
+        const int64_t top = last_word + 3;                                   // last_word is a word's first byte
+        begin = begin < 0 ? 0 : (begin > top ? top : begin);
+        lowest = lowest < 0 ? 0 : (lowest > top ? top : lowest);
         const uint32_t skip = (uint32_t)begin & 3u;
         const int64_t first_word = begin - skip;
-        // the descriptor starts at the first word of the wavefront's first active lane; a lane
-        // whose stream lies before it or 4 GiB behind it gets an offset that wraps, which
-        // reads zeros or some other place inside the buffer
-        const uint32_t org_lo = __builtin_amdgcn_readfirstlane((uint32_t)first_word);
-        const uint32_t org_hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)first_word >> 32));
+        // the descriptor starts at the word of the wavefront's lowest stream, so every lane's
+        // offset from it is its own distance; one that is 4 GiB or more wraps, which reads zeros
+        // or some other place inside the buffer
+        const int64_t low_word = lowest & ~3ll;
+        const uint32_t org_lo = __builtin_amdgcn_readfirstlane((uint32_t)low_word);
+        const uint32_t org_hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)low_word >> 32));
         const int64_t origin = (int64_t)(((uint64_t)org_hi << 32) | org_lo);
         const int64_t room = last_word + 4 - origin;                           // >= 4
         rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(window + origin), 0,
@@ -379,16 +383,25 @@ __global__ __launch_bounds__(BS) void decode_streams_kernel(DecodeArgs a)
         }
     }
     special = __syncthreads_or(special);
-    if (!id.active) return;
 
     const int64_t stream = (id.sub * a.sg.rows + id.row) * a.sg.nc + id.ch;
-    int64_t begin;
-    if (SRC == SRC_OFFSETS) begin = a.offsets[stream];
-    else if (SRC == SRC_PREFIX) begin = stream ? a.offsets[stream - 1] : 0;
-    else begin = id.row * a.p0 + id.ch * a.p1;
+    int64_t begin = INT64_MAX;
+    if (id.active) {
+        if (SRC == SRC_OFFSETS) begin = a.offsets[stream];
+        else if (SRC == SRC_PREFIX) begin = stream ? a.offsets[stream - 1] : 0;
+        else begin = id.row * a.p0 + id.ch * a.p1;
+    }
+    // the lowest stream start of the wavefront, taken while all of its lanes are still here
+    int64_t lowest = begin;
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) {
+        const int64_t other = __shfl_xor(lowest, o, 64);
+        lowest = other < lowest ? other : lowest;
+    }
+    if (!id.active) return;
 
     DecodeLane s;
-    s.off = s.rd.start(a.bytes, a.last_word, begin + a.bytes_skew);
+    s.off = s.rd.start(a.bytes, a.last_word, begin + a.bytes_skew, lowest + a.bytes_skew);
     s.low = 0;
     s.span = 0;                        // span modulo 2^32: 0 is the full range (see RangeEncoder)
     s.colp = (lds_char *)(rows + 2 * tid);

@@ -190,3 +190,35 @@ def test_streams_that_begin_in_the_last_word_of_an_exact_size_buffer(oracle, nt)
         tac.decode_fast_prefsum(torch.from_numpy(cdf.view(np.int16)).to(DEV), base[shift:],
                                 torch.from_numpy(prefix).to(DEV), out)
         assert np.array_equal(out.cpu().numpy(), sym), shift
+
+
+def test_streams_with_bogus_offsets_do_not_disturb_their_neighbours():
+    """Offsets that are not running sums of the lengths (negative, beyond the payload, beyond
+    4 GiB, or simply another stream's) make their own streams decode to garbage; every other
+    stream, including those in the same wavefront, still decodes as before, and nothing is
+    read outside the payload (the kernel reads it through a range-checked descriptor)."""
+    codec, _ = _mods()
+    L, T, H, D = 2, 256, 2, 64
+    C = H * D
+    g = torch.Generator().manual_seed(5)
+    kv = (torch.randn(L, 2, T, H, D, generator=g) * torch.rand(C, generator=g).reshape(H, D)).to(torch.float16).to(DEV)
+    bins = torch.tensor([32.0, 16.0])
+    enc = codec.encode_kv(kv, bins, bins, chunk_tokens=256)
+    clean = codec.decode_encoded(enc, bins, bins, out_dtype=torch.float16)
+    nstreams = 2 * L * C
+    total = int(enc.offsets[-1])
+    rng = np.random.default_rng(11)
+    bad = np.unique(np.concatenate([[0, 64, 65, 127, 128, nstreams - 1], rng.integers(0, nstreams, 40)]))
+    bogus = np.concatenate([[-5, -10 ** 12, 10 ** 12, (1 << 32) + 7, total + 100, total, total - 1],
+                            rng.integers(0, total, bad.size)])[:bad.size]
+    offsets = enc.offsets.clone()
+    offsets[torch.from_numpy(bad).to(DEV)] = torch.from_numpy(bogus.astype(np.int64)).to(DEV)
+    out = codec.decode_kv(enc.cdf, enc.maxima, offsets, enc.payload[:total].clone(), bins, bins, L, T, H, D, 256,
+                          out_dtype=torch.float16)
+    torch.cuda.synchronize()
+    keep = torch.ones(nstreams, dtype=torch.bool)
+    keep[torch.from_numpy(bad)] = False
+    # stream (row = kv * L + l, channel) is out[l, kv, :, channel]
+    got = out.reshape(L, 2, T, C).permute(1, 0, 3, 2).reshape(nstreams, T).cpu()
+    want = clean.reshape(L, 2, T, C).permute(1, 0, 3, 2).reshape(nstreams, T).cpu()
+    assert torch.equal(got[keep].view(torch.int16), want[keep].view(torch.int16))

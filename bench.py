@@ -3,8 +3,8 @@
 
 A step is one encode of the whole synthetic KV cache followed by one decode of the
 result, inputs and outputs resident in HBM, every buffer allocated before the timed
-region.  Prints ONE JSON line.  Workload (default): the Mistral-7B-shape cache of
-BASELINE.json configs[1]: 32 layers x {K,V} x 8192 tokens x 8 heads x 128, fp16, one
+region.  Prints ONE JSON line.  Workload (default, "config2"): a Mistral-7B-shape
+cache, 32 layers x {K,V} x 8192 tokens x 8 heads x 128, fp16, one
 table per 256-token chunk, reference 7B bins table.
 """
 import argparse
@@ -21,7 +21,7 @@ HBM_PEAK_GBPS = 8000.0
 
 # HBM bytes per launch of decode_streams_kernel measured with rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE (two runs, each scaled by what the same counter reads for a plain conversion
-# kernel of known size: x2.000 and x1.000): 310.4 MB read + 1073.7 MB written.  A profile
+# kernel of known size: x2.000 and x1.000): 292.4 MB read + 1073.7 MB written.  A profile
 # measurement of this workload, not something this script can observe while it runs.
 MEASURED_DECODE_TRAFFIC_BYTES = {"config2": 1366.1e6}
 

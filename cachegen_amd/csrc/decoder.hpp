@@ -36,14 +36,21 @@ namespace {
 // GPUs: 32-bit data format, everything else off.
 constexpr int kBufferWord3 = 0x00020000;
 
+// The most bits one symbol can move for a table without zero-width entries.
+constexpr uint32_t kSymbolBits = 18;
+
 struct BitReader {
     // Words are fetched with buffer loads: the descriptor (uniform over the wavefront) covers
     // the byte buffer from the wavefront's first stream to its last readable word, a lane
     // addresses it with a 32-bit offset, and a load outside it returns zero instead of faulting.
     __amdgpu_buffer_rsrc_t rsrc;
     uint32_t pos;            // byte offset inside the descriptor's range of the next word to fetch
-    uint64_t win;            // the next `avail` bits of the stream, left-aligned, zeros below
-    int avail;
+    uint64_t win;            // the unread bits of the stream that are loaded, left-aligned, zeros below
+    // how many bits `win` holds beyond kSymbolBits, the most one symbol can take: counted this
+    // way, the subtraction that consumes a symbol's bits borrows exactly when the window no
+    // longer covers another symbol, and that borrow is the test
+    uint32_t spare;
+    bool short_of_bits;      // the last shift_in left fewer than kSymbolBits
     uint32_t nextw;          // the word after the window, as loaded
 
     __device__ __forceinline__ uint32_t raw()
@@ -83,28 +90,29 @@ struct BitReader {
         const uint64_t head = (((uint64_t)b0 << 32) | b1) << s;
         const uint64_t rest = (((uint64_t)b1 << 32) | b2) << s;
         win = rest;
-        avail = 64 - (int)s;
+        spare = 64u - kSymbolBits - s;
+        short_of_bits = false;
         return (uint32_t)(head >> 32);
     }
 
-    // off = (off << n) | next n bits, 0 <= n <= 31 and n <= avail
+    // off = (off << n) | next n bits, 0 <= n <= 31 and n <= spare + kSymbolBits
     __device__ __forceinline__ uint32_t shift_in(uint32_t off, int n)
     {
         // two 64-bit shifts: {off, top word of the window} and the window itself
         const uint64_t pair = (((uint64_t)off << 32) | (uint32_t)(win >> 32)) << n;
         off = (uint32_t)(pair >> 32);
         win <<= n;
-        avail -= n;
+        short_of_bits = __builtin_usub_overflow(spare, (uint32_t)n, &spare);
         return off;
     }
 
     // brings the window to more than 32 bits
     __device__ __forceinline__ void top_up()
     {
-        if (avail <= 32) {                      // the low word is empty
-            const uint64_t in = (((uint64_t)__builtin_bswap32(nextw)) << 32) >> (avail & 63);
+        if ((int32_t)spare <= 32 - (int)kSymbolBits) {          // at most 32 bits: the low word is empty
+            const uint64_t in = (((uint64_t)__builtin_bswap32(nextw)) << 32) >> ((spare + kSymbolBits) & 63);
             win = (((win >> 32) | (in >> 32)) << 32) | (uint32_t)in;
-            avail += 32;
+            spare += 32;
             nextw = raw();
         }
     }
@@ -334,7 +342,7 @@ __device__ __forceinline__ void decode_lane(const DecodeArgs &a, DecodeLane &s, 
             const int i = i0 + j;
             if (i >= n) break;
             if (j == 0) s.rd.top_up();
-            else if (__builtin_expect(s.rd.avail < 18, 0)) s.rd.top_up();
+            else if (__builtin_expect(s.rd.short_of_bits, 0)) s.rd.top_up();
             decode_symbol<BS, LOG2, OUT, SKIP, SAFE>(a, s, lp, nsteps, rm[j], i, i == n - 1);
         }
     }

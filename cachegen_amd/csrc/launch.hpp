@@ -82,6 +82,10 @@ int launch_scan(const int32_t *lengths, int64_t n, int32_t clamp, int64_t *offse
 {
     const int64_t ntiles = ceil_div(n, kScanTile);
     int64_t *sums = static_cast<int64_t *>(scratch);
+    if (ntiles == 1) {
+        scan_apply_kernel<<<dim3(1), dim3(kScanThreads), 0, stream>>>(lengths, n, clamp, nullptr, offsets);
+        return check_launch("scan_lengths");
+    }
     scan_tile_sums_kernel<<<dim3((unsigned)ntiles), dim3(kScanThreads), 0, stream>>>(lengths, n, clamp, sums);
     scan_sums_kernel<<<dim3(1), dim3(kScanThreads), 0, stream>>>(sums, ntiles);
     scan_apply_kernel<<<dim3((unsigned)ntiles), dim3(kScanThreads), 0, stream>>>(lengths, n, clamp, sums, offsets);

@@ -101,7 +101,8 @@ __global__ __launch_bounds__(kScanThreads) void scan_apply_kernel(
         s += x;
     }
     int64_t total;
-    int64_t run = sums[blockIdx.x] + block_exclusive_scan(s, lds, total);
+    // sums == nullptr: the input is a single tile and this kernel is the whole scan
+    int64_t run = (sums ? sums[blockIdx.x] : 0) + block_exclusive_scan(s, lds, total);
     for (int j = 0; j < kScanPerThread; ++j) {
         if (base + j < n) offsets[base + j] = run;
         run += v[j];

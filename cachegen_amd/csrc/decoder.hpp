@@ -41,7 +41,7 @@ constexpr uint32_t kSymbolBits = 18;
 
 struct BitReader {
     // Words are fetched with buffer loads: the descriptor (uniform over the wavefront) covers
-    // the byte buffer from the wavefront's first stream to its last readable word, a lane
+    // the byte buffer from the wavefront's lowest stream to its last readable word, a lane
     // addresses it with a 32-bit offset, and a load outside it returns zero instead of faulting.
     __amdgpu_buffer_rsrc_t rsrc;
     uint32_t pos;            // byte offset inside the descriptor's range of the next word to fetch

@@ -159,12 +159,11 @@ __device__ __forceinline__ uint32_t lds_entry(lds_char *p, int byte_offset)
     return *(lds_u16 *)(p + byte_offset);
 }
 
-// float32 -> bfloat16 bits, round to nearest even, for anything but a NaN
-__device__ __forceinline__ uint32_t float_to_bf16_bits_no_nan(float f)
+// float32 -> bfloat16 bits by the hardware's conversion (round to nearest even, a NaN stays
+// a NaN): one instruction on this GPU
+__device__ __forceinline__ uint32_t float_to_bf16_bits_hw(float f)
 {
-    uint32_t u = __float_as_uint(f);
-    u += 0x7FFFu + ((u >> 16) & 1u);
-    return u >> 16;
+    return __builtin_bit_cast(uint16_t, (__bf16)f);
 }
 
 struct DecodeLane {
@@ -293,7 +292,7 @@ __device__ __forceinline__ void decode_symbol(const DecodeArgs &a, DecodeLane &s
             s.phase = s.phase + 1 == a.delta_group ? 0 : s.phase + 1;
         }
         uint32_t bits;
-        if (OUT == OUT_BF16) bits = SAFE ? float_to_bf16_bits(v) : float_to_bf16_bits_no_nan(v);
+        if (OUT == OUT_BF16) bits = float_to_bf16_bits_hw(v);
         else bits = float_to_f16_bits(v);
         __builtin_amdgcn_raw_buffer_store_b16((short)bits, s.orsrc, (int)s.ovoff, (int)((uint32_t)i * (uint32_t)a.ot * 2u), 0);
     }

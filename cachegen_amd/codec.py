@@ -75,7 +75,11 @@ class EncodedKV:
         return int(self.offsets[-1].item())
 
     def check(self):
-        st = int(self.status.item())
+        self.raise_for_status(int(self.status.item()))
+
+    @staticmethod
+    def raise_for_status(st):
+        """st: the status word as read back from the device."""
         if st & 1:
             raise RuntimeError("a stream exceeded %d bytes (the reference overruns its buffer there)"
                                % MAX_TOKENS_PER_STREAM)

@@ -271,37 +271,55 @@ def _stream():
     return torch.cuda.current_stream().cuda_stream
 
 
-def _device_counts(cdf, tokens):
-    """Device form of tables_to_counts + pack_counts for cdf int16 [nchunks, 2L, C, Lp]:
-    (nsym list per (chunk, row), ragged count bytes uint8 on the device) or None if some table is
-    not the table of a histogram."""
+def _device_counts_launch(cdf, tokens):
+    """First half of the device form of tables_to_counts + pack_counts for cdf int16
+    [nchunks, 2L, C, Lp]: launches the conversion and returns (dense counts uint8 [G, C, Lp-1],
+    nsym int32 [G], inexact int32 [1]), all still on the device and not waited for."""
     import torch
     from .. import _lib
     nchunks, rows, C, lp = cdf.shape
     G = nchunks * rows
     dev = cdf.device
     cdf = cdf.contiguous()
-    tok = torch.tensor([t for t in tokens for _ in range(rows)], dtype=torch.int32, device=dev)
+    tok = torch.tensor([t for t in tokens for _ in range(rows)], dtype=torch.int32).to(dev, non_blocking=True)
     dense = torch.empty((G, C, lp - 1), dtype=torch.uint8, device=dev)
     nsym = torch.empty(G, dtype=torch.int32, device=dev)
     inexact = torch.empty(1, dtype=torch.int32, device=dev)
-    lib = _lib.lib()
     with torch.cuda.device(dev):
-        _lib.check(lib.cg_tables_to_counts(cdf.data_ptr(), lp - 1, G, C, tok.data_ptr(), dense.data_ptr(),
-                                           nsym.data_ptr(), inexact.data_ptr(), _stream()))
-        host = torch.cat([nsym, inexact]).tolist()
-        if host[-1]:
-            return None
-        ks = host[:-1]
-        starts, total = [], 0
-        for k in ks:
-            starts.append(total)
-            total += C * k
-        data = torch.empty(total, dtype=torch.uint8, device=dev)
-        d_starts = torch.tensor(starts, dtype=torch.int64, device=dev)
-        _lib.check(lib.cg_pack_counts(dense.data_ptr(), lp - 1, G, C, nsym.data_ptr(), d_starts.data_ptr(),
-                                      data.data_ptr(), _stream()))
-    return ks, data
+        _lib.check(_lib.lib().cg_tables_to_counts(cdf.data_ptr(), lp - 1, G, C, tok.data_ptr(), dense.data_ptr(),
+                                                  nsym.data_ptr(), inexact.data_ptr(), _stream()))
+    return dense, nsym, inexact
+
+
+def _device_counts_finish(dense, nsym, ks):
+    """Second half: ks is nsym read back on the host; returns the ragged count bytes uint8 on
+    the device."""
+    import torch
+    from .. import _lib
+    G, C, nb = dense.shape
+    dev = dense.device
+    starts, total = [], 0
+    for k in ks:
+        starts.append(total)
+        total += C * k
+    data = torch.empty(total, dtype=torch.uint8, device=dev)
+    d_starts = torch.tensor(starts, dtype=torch.int64).to(dev, non_blocking=True)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().cg_pack_counts(dense.data_ptr(), nb, G, C, nsym.data_ptr(), d_starts.data_ptr(),
+                                             data.data_ptr(), _stream()))
+    return data
+
+
+def _device_counts(cdf, tokens):
+    """Device form of tables_to_counts + pack_counts for cdf int16 [nchunks, 2L, C, Lp]:
+    (nsym list per (chunk, row), ragged count bytes uint8 on the device) or None if some table is
+    not the table of a histogram."""
+    import torch
+    dense, nsym, inexact = _device_counts_launch(cdf, tokens)
+    host = torch.cat([nsym, inexact]).tolist()
+    if host[-1]:
+        return None
+    return host[:-1], _device_counts_finish(dense, nsym, host[:-1])
 
 
 def _device_tables(nsym_host, nsym_dev, data, C, lp, tokens):
@@ -342,32 +360,48 @@ def pack_chunks(enc, first_chunk: int = 0, num_chunks: Optional[int] = None, per
         num_chunks = nch - first_chunk
     if first_chunk < 0 or num_chunks <= 0 or first_chunk + num_chunks > nch:
         raise ValueError("chunk range outside the encoded tensor")
-    enc.check()
     L, H, D, S, T = enc.num_layers, enc.num_heads, enc.head_size, enc.chunk_tokens, enc.num_tokens
     C = H * D
     spc = enc.subchunks_per_chunk
-    bounds = enc.sub_boundaries()
     bf16 = enc.maxima.dtype == torch.bfloat16
     groups = [(c, c + 1) for c in range(first_chunk, first_chunk + num_chunks)] if per_chunk \
         else [(first_chunk, first_chunk + num_chunks)]
     all_tokens = chunk_token_counts(T, S)
+    c0, c1 = first_chunk, first_chunk + num_chunks
+
+    # everything the host has to know before it can lay the blobs out, read back at once:
+    # status word, payload offset at every sub-chunk boundary, smallest and largest stream
+    # length, and (compact) the symbol count of every table plus the flag that says whether
+    # all tables are tables of histograms
+    dev = enc.payload.device
+    nsub = enc.lengths.shape[0]
+    idx = torch.arange(0, nsub + 1, device=dev) * (2 * L * C)
+    want_counts = compact and S <= MAX_STREAM_BYTES
+    parts = [enc.status.to(torch.int64).reshape(1), enc.offsets[idx]]
+    if compact:
+        parts += [enc.lengths.min().to(torch.int64).reshape(1), enc.lengths.max().to(torch.int64).reshape(1)]
+    if want_counts:
+        dense, nsym_dev, inexact = _device_counts_launch(enc.cdf[c0:c1], all_tokens[c0:c1])
+        parts += [inexact.to(torch.int64), nsym_dev.to(torch.int64)]
+    meta = torch.cat(parts).tolist()
+    enc.raise_for_status(meta[0])
+    bounds = meta[1:nsub + 2]
+    rest = meta[nsub + 2:]
 
     version, flags, lengths_src = VERSION, 0, enc.lengths
     packed = None                       # (nsym [nch, 2L], data, byte offset of every (chunk, row) in data)
     if compact:
         version = VERSION_COMPACT
-        c0, c1 = first_chunk, first_chunk + num_chunks
-        if S <= MAX_STREAM_BYTES:
-            got = _device_counts(enc.cdf[c0:c1], all_tokens[c0:c1])
-            if got is not None:
-                ks, data = got                                   # nsym per (chunk, row), ragged count bytes
-                starts = [0]
-                for k in range(c1 - c0):
-                    starts.append(starts[-1] + C * sum(ks[k * 2 * L:(k + 1) * 2 * L]))
-                nsym = torch.tensor(ks, dtype=torch.uint8, device=data.device).view(c1 - c0, 2 * L)
-                packed = (nsym, data, starts)
-                flags |= FLAG_COUNT_TABLES
-        lo, hi = torch.stack([enc.lengths.min(), enc.lengths.max()]).tolist()
+        lo, hi = rest[0], rest[1]
+        if want_counts and not rest[2]:
+            ks = rest[3:]                                        # nsym per (chunk, row)
+            data = _device_counts_finish(dense, nsym_dev, ks)    # ragged count bytes
+            starts = [0]
+            for k in range(c1 - c0):
+                starts.append(starts[-1] + C * sum(ks[k * 2 * L:(k + 1) * 2 * L]))
+            nsym = nsym_dev.to(torch.uint8).view(c1 - c0, 2 * L)
+            packed = (nsym, data, starts)
+            flags |= FLAG_COUNT_TABLES
         if lo >= 0 and hi <= 0xFFFF:
             lengths_src = enc.lengths.to(torch.int16)         # bit pattern of the uint16 value
             flags |= FLAG_LENGTHS_U16
@@ -388,7 +422,6 @@ def pack_chunks(enc, first_chunk: int = 0, num_chunks: Optional[int] = None, per
                             version, flags, tables_bytes or 0)
         plans.append((total, geo, head, (c0, c1, t0, t1, g0, g1)))
         total += geo["total"][0]
-    dev = enc.payload.device
     stage = torch.zeros(total, dtype=torch.uint8, device=dev)
     heads = torch.frombuffer(bytearray(b"".join(p[2] for p in plans)), dtype=torch.uint8).to(dev)
 

@@ -102,15 +102,16 @@ class CacheGenDeserializer(Deserializer):
                                encoder_output.head_size, chunk_tokens=ntokens, fmt=self.fmt, out=out)
 
     def _from_flat(self, bs, out=None) -> torch.Tensor:
-        h, cdf, maxima, lengths, payload = wire.unpack_to_device(bs, self.key_bins.device)
+        # the container's own consistency (stream lengths against the payload size) is checked on
+        # the host inside unpack_to_device; the decode is queued before anything waits for the device
+        h, cdf, maxima, lengths, payload = wire.unpack_to_device(bs, self.key_bins.device, defer_checks=True)
         if h["num_layers"] != self.key_bins.numel():
             raise ValueError("blob has %d layers, this deserializer's model %d"
                              % (h["num_layers"], self.key_bins.numel()))
         offsets = codec.scan_lengths(lengths)
-        total, shortest = torch.stack([offsets[-1], lengths.min().to(torch.int64)]).tolist()
-        if total != h["payload_bytes"] or shortest < 0:
-            raise ValueError("wire container: payload size is not the sum of the stream lengths")
-        return codec.decode_kv(cdf, maxima, offsets, payload, self.key_bins, self.value_bins,
-                               h["num_layers"], h["num_tokens"], h["num_heads"], h["head_size"],
-                               chunk_tokens=h["chunk_tokens"], fmt=self.fmt, delta_group=h["delta_group"],
-                               out=out)
+        result = codec.decode_kv(cdf, maxima, offsets, payload, self.key_bins, self.value_bins,
+                                 h["num_layers"], h["num_tokens"], h["num_heads"], h["head_size"],
+                                 chunk_tokens=h["chunk_tokens"], fmt=self.fmt, delta_group=h["delta_group"],
+                                 out=out)
+        h["check"]()
+        return result

@@ -322,10 +322,16 @@ def _device_counts(cdf, tokens):
     return host[:-1], _device_counts_finish(dense, nsym, host[:-1])
 
 
-def _device_tables(nsym_host, nsym_dev, data, C, lp, tokens):
+def _raise_if_invalid_counts(invalid):
+    if int(invalid.item()):
+        raise ValueError("wire container: histogram counts do not add up to the chunk's tokens")
+
+
+def _device_tables(nsym_host, nsym_dev, data, C, lp, tokens, defer=False):
     """Device form of unpack_counts + counts_to_tables -> cdf int16 [nchunks, 2L, C, Lp].
     nsym_host: numpy uint8 [nchunks, 2L] (read from the blob on the host), nsym_dev the same bytes
-    on the device."""
+    on the device.  defer: do not wait for the kernel's verdict on the counts; returns
+    (cdf, check) where check() waits and raises."""
     import torch
     from .. import _lib
     nchunks, rows = nsym_host.shape
@@ -343,8 +349,9 @@ def _device_tables(nsym_host, nsym_dev, data, C, lp, tokens):
         _lib.check(_lib.lib().cg_counts_to_tables(data.data_ptr(), data.numel(), lp - 1, G, C, tok.data_ptr(),
                                                   nsym_dev.data_ptr(), small.data_ptr(), cdf.data_ptr(),
                                                   invalid.data_ptr(), _stream()))
-    if int(invalid.item()):
-        raise ValueError("wire container: histogram counts do not add up to the chunk's tokens")
+    if defer:
+        return cdf, (lambda: _raise_if_invalid_counts(invalid))
+    _raise_if_invalid_counts(invalid)
     return cdf
 
 
@@ -448,10 +455,13 @@ def pack_chunks(enc, first_chunk: int = 0, num_chunks: Optional[int] = None, per
     return [raw[base:base + geo["total"][0]].tobytes() for base, geo, _, _ in plans]
 
 
-def unpack_to_device(blob, device):
+def unpack_to_device(blob, device, defer_checks=False):
     """-> (header dict, cdf, maxima, lengths, payload) on the device, which the blob reached in a
     single copy from pinned host memory: views of that buffer where the stored form is the
-    tensor itself, rebuilt tensors where it is not (version 2)."""
+    tensor itself, rebuilt tensors where it is not (version 2).  The stream lengths are checked
+    against the payload size on the host.  defer_checks: nothing here waits for the device; the
+    header dict then holds "check", to be called once the caller has queued its own work: it
+    waits for the device and raises what the device-side checks found."""
     import torch
     h = read_header(blob)
     geo = h["geometry"]
@@ -459,7 +469,14 @@ def unpack_to_device(blob, device):
     lp, nchunks = h["max_bins"] + 1, geo["nchunks"][0]
     host = torch.empty(len(blob), dtype=torch.uint8, pin_memory=True)
     host.numpy()[:] = np.frombuffer(blob, dtype=np.uint8)
-    buf = host.to(device, non_blocking=False)
+    buf = host.to(device, non_blocking=False)      # waits: the pinned buffer is free for the next call at once
+    # the lengths are in the blob: their sum is checked here, without asking the device
+    off, size = geo["lengths"]
+    host_lengths = np.frombuffer(blob, dtype=np.uint16 if h["lengths_u16"] else np.int32, count=h["nsub"] * 2 * L * C,
+                                 offset=off)
+    if int(host_lengths.sum(dtype=np.int64)) != h["payload_bytes"] or (host_lengths.size and int(host_lengths.min()) < 0):
+        raise ValueError("wire container: payload size is not the sum of the stream lengths")
+    h["check"] = lambda: None
 
     def section(name, dtype, shape):
         off, size = geo[name]
@@ -473,7 +490,9 @@ def unpack_to_device(blob, device):
         if int(nsym_host.min()) < 1 or int(nsym_host.max()) > lp - 1:
             raise ValueError("wire container: symbol count outside the table")
         cdf = _device_tables(nsym_host, raw[:nchunks * 2 * L], raw[nchunks * 2 * L:], C, lp,
-                             chunk_token_counts(T, h["chunk_tokens"]))
+                             chunk_token_counts(T, h["chunk_tokens"]), defer=defer_checks)
+        if defer_checks:
+            cdf, h["check"] = cdf
     else:
         cdf = section("cdf", torch.int16, (nchunks, 2 * L, C, lp))
     maxima = section("maxima", torch.bfloat16 if h["bf16_maxima"] else torch.float16, (2, L, T))

@@ -367,8 +367,20 @@ __global__ __launch_bounds__(BS) void decode_streams_kernel(DecodeArgs a)
         const int64_t nvalid = (a.sg.nc - ch0 < BS) ? (a.sg.nc - ch0) : BS;
         const int total = (int)nvalid * lp;
         TableWalk w(tid, BS, lp);
-        for (int i = tid; i < total; i += BS, w.next(lp))
-            *reinterpret_cast<uint16_t *>(rows + w.e * kRow + 2 * w.c) = w.e == 0 ? (uint16_t)0 : src[i];
+        // sixteen loads are issued before the first value is needed: one trip to memory per
+        // sixteen table entries of a lane instead of one per entry
+        constexpr int kBatch = 16;
+        for (int i0 = tid; i0 < total; i0 += kBatch * BS) {
+            uint16_t v[kBatch];
+#pragma unroll
+            for (int j = 0; j < kBatch; ++j) v[j] = i0 + j * BS < total ? src[i0 + j * BS] : (uint16_t)0;
+#pragma unroll
+            for (int j = 0; j < kBatch; ++j) {
+                if (i0 + j * BS < total)
+                    *reinterpret_cast<uint16_t *>(rows + w.e * kRow + 2 * w.c) = w.e == 0 ? (uint16_t)0 : v[j];
+                w.next(lp);
+            }
+        }
     }
     int64_t kvi = 0, l = 0;
     int special = 0;                   // a row maximum that is infinite or NaN

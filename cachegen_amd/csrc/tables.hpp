@@ -102,8 +102,17 @@ __device__ __forceinline__ void stage_tables16(uint16_t *tab, const uint16_t *cd
     const int64_t nvalid = (nc - ch0 < BS) ? (nc - ch0) : BS;
     const int total = (int)nvalid * lp;
     TableWalk w(threadIdx.x, BS, lp);
-    for (int i = threadIdx.x; i < total; i += BS, w.next(lp)) {
-        tab[w.e * TableStride<BS>::k16 + w.c] = cdf[i];
+    // sixteen loads in flight at a time: one trip to memory per sixteen entries of a lane
+    constexpr int kBatch = 16;
+    for (int i0 = threadIdx.x; i0 < total; i0 += kBatch * BS) {
+        uint16_t v[kBatch];
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j) v[j] = i0 + j * BS < total ? cdf[i0 + j * BS] : (uint16_t)0;
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j) {
+            if (i0 + j * BS < total) tab[w.e * TableStride<BS>::k16 + w.c] = v[j];
+            w.next(lp);
+        }
     }
 }
 

@@ -25,6 +25,12 @@ HBM_PEAK_GBPS = 8000.0
 # measurement of this workload, not something this script can observe while it runs.
 MEASURED_DECODE_TRAFFIC_BYTES = {"config2": 1366.1e6}
 
+# VALU wave-instructions per launch of decode_streams_kernel (rocprofv3 --pmc SQ_INSTS_VALU, same
+# profile).  The kernel's own limit is the issue of these: one per 4 cycles per SIMD for most
+# of them, 1024 SIMDs, at the clock the profile's GRBM_GUI_ACTIVE gives (2.3 GHz).
+MEASURED_DECODE_VALU_INSTS = {"config2": 387.26e6}
+VALU_ISSUE_PER_SECOND = 1024 * 2.3e9 / 4
+
 WORKLOADS = {
     # name: (layers, tokens, heads, head_size, chunk_tokens, model name for the bins table, seed)
     "config1": (2, 512, 8, 64, 512, None, 1235),
@@ -297,6 +303,15 @@ def main():
             "avg_launch_ms": round(dec_avg, 4),
         },
     }
+    if args.workload in MEASURED_DECODE_VALU_INSTS:
+        insts = MEASURED_DECODE_VALU_INSTS[args.workload]
+        result["valu_issue"] = {
+            "kernel": "decode_streams_kernel",
+            "insts_per_launch": insts,
+            "insts_per_symbol_and_lane": round(insts * 64 / (kv_bytes / 2), 1),
+            "frac_of_issue_rate": round(insts / (dec_avg * 1e-3) / VALU_ISSUE_PER_SECOND, 3),
+            "note": "profile counter x live duration; above 1 where cheap instructions issue in under 4 cycles",
+        }
     # what one chunk weighs on the wire in the two flat containers (first chunk, vllm layout only)
     if fmt == "vllm":
         from cachegen_amd.serde import wire

@@ -206,26 +206,33 @@ int set_byte_window(DecodeArgs &a, const uint8_t *bytes, int64_t nbytes, const c
 
 size_t decode_shmem(int lp, int block) { return align_up((size_t)lp * block * sizeof(uint16_t), 4) + (size_t)(lp + kSub) * sizeof(float); }
 
+// Tables of 2^k symbols (lp = 2^k + 1) take the kernel with the unrolled search.
+template <int BS, int SRC, int OUT>
+void launch_decode_log2(const DecodeArgs &a, dim3 grid, size_t shmem, hipStream_t stream)
+{
+    const dim3 blk(BS);
+    switch (a.lp) {
+    case 9: decode_streams_kernel<BS, 3, SRC, OUT><<<grid, blk, shmem, stream>>>(a); break;
+    case 17: decode_streams_kernel<BS, 4, SRC, OUT><<<grid, blk, shmem, stream>>>(a); break;
+    case 33: decode_streams_kernel<BS, 5, SRC, OUT><<<grid, blk, shmem, stream>>>(a); break;
+    case 65: decode_streams_kernel<BS, 6, SRC, OUT><<<grid, blk, shmem, stream>>>(a); break;
+    default: decode_streams_kernel<BS, -1, SRC, OUT><<<grid, blk, shmem, stream>>>(a); break;
+    }
+}
+
 template <int SRC>
 int launch_decode_symbols(const DecodeArgs &a, int64_t nblocks, int block, hipStream_t stream)
 {
-    const dim3 grid((unsigned)nblocks), blk(block);
+    const dim3 grid((unsigned)nblocks);
     const size_t shmem = decode_shmem(a.lp, block);
-    CG_DISPATCH_BS(block, (decode_streams_kernel<BS, -1, SRC, OUT_SYMBOLS><<<grid, blk, shmem, stream>>>(a)));
+    CG_DISPATCH_BS(block, (launch_decode_log2<BS, SRC, OUT_SYMBOLS>(a, grid, shmem, stream)));
     return check_launch("decode");
 }
 
 template <int BS, int OUT>
 void launch_decode_kv_log2(const DecodeArgs &a, dim3 grid, size_t shmem, hipStream_t stream)
 {
-    const dim3 blk(BS);
-    switch (a.lp) {
-    case 9: decode_streams_kernel<BS, 3, SRC_OFFSETS, OUT><<<grid, blk, shmem, stream>>>(a); break;
-    case 17: decode_streams_kernel<BS, 4, SRC_OFFSETS, OUT><<<grid, blk, shmem, stream>>>(a); break;
-    case 33: decode_streams_kernel<BS, 5, SRC_OFFSETS, OUT><<<grid, blk, shmem, stream>>>(a); break;
-    case 65: decode_streams_kernel<BS, 6, SRC_OFFSETS, OUT><<<grid, blk, shmem, stream>>>(a); break;
-    default: decode_streams_kernel<BS, -1, SRC_OFFSETS, OUT><<<grid, blk, shmem, stream>>>(a); break;
-    }
+    launch_decode_log2<BS, SRC_OFFSETS, OUT>(a, grid, shmem, stream);
 }
 
 }  // namespace

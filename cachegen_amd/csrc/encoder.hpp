@@ -153,14 +153,15 @@ struct RangeEncoder {
         // the upper bound of symbol smax is 2^16 and not the table's last entry; shifted left
         // by 16 that is 0 modulo 2^32, and T(2^16) is the span
         const bool top = SENTINEL && s == smax;
-        uint32_t t_lo, width;
+        // T(c) = (span * c) >> 16 = high word of span * (c << 16)
+        uint32_t t_lo = __umulhi(span, bound_lo);
+        uint32_t width = (top ? span : __umulhi(span, bound_hi)) - t_lo;
         if (__builtin_expect(span == 0, 0)) {
-            t_lo = bound_lo;                                // c << 16
+            // the full range: T(c) = c << 16.  The empty statement makes the compiler jump over
+            // this block when no lane needs it instead of issuing it with every lane masked off.
+            asm volatile("");
+            t_lo = bound_lo;
             width = (top ? 0u : bound_hi) - bound_lo;
-        } else {
-            // T(c) = (span * c) >> 16 = high word of span * (c << 16)
-            t_lo = __umulhi(span, bound_lo);
-            width = (top ? span : __umulhi(span, bound_hi)) - t_lo;
         }
         low += t_lo;
         const uint32_t high = low + width - 1u;

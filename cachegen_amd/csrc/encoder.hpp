@@ -29,8 +29,10 @@ struct BitWriter {
     int wstride;            // bytes from one word of the stream to the next (4: contiguous)
     int cap;
     int nbytes;
-    uint64_t acc;           // the low `nacc` bits are waiting to be written; bits above are stale
-    int nacc;
+    uint64_t acc;           // the low 64 - room bits are waiting to be written; bits above are stale
+    // free bits of the accumulator: counted this way, the subtraction that books a put borrows
+    // exactly when the bits do not fit, and that borrow is the test
+    uint32_t room;
 
     // the last words of a stream that does not fit its slot: keep what fits
     __device__ __forceinline__ void store_clipped(uint32_t word)
@@ -60,9 +62,9 @@ struct BitWriter {
     // write one word if 32 bits are waiting
     __device__ __forceinline__ void flush_word()
     {
-        if (nacc >= 32) {
-            store_word((uint32_t)(acc >> (nacc - 32)));
-            nacc -= 32;
+        if (room <= 32u) {
+            store_word((uint32_t)(acc >> (32u - room)));
+            room += 32u;
         }
     }
 
@@ -71,9 +73,13 @@ struct BitWriter {
     template <bool ROOM = false>
     __device__ __forceinline__ void put(uint32_t v, int m)
     {
-        if (!ROOM && __builtin_expect(nacc + m > 64, 0)) flush_word();   // more than 32 are waiting then
+        uint32_t left;
+        if (__builtin_expect(__builtin_usub_overflow(room, (uint32_t)m, &left), 0) && !ROOM) {
+            flush_word();                                  // more than 32 bits were waiting
+            left = room - (uint32_t)m;
+        }
+        room = left;
         acc = (acc << m) | v;
-        nacc += m;
     }
 
     // one bit, then `count` copies of its complement (any count): the general form of
@@ -98,6 +104,7 @@ struct BitWriter {
     {
         flush_word();
         flush_word();
+        const int nacc = 64 - (int)room;
         if (nacc > 0) {
             uint32_t r = (uint32_t)(acc << (32 - nacc));
             for (int left = nacc, j = 0; left > 0; left -= 8, ++j) {
@@ -138,7 +145,7 @@ struct RangeEncoder {
         w.cap = cap;
         w.nbytes = 0;
         w.acc = 0;
-        w.nacc = 0;
+        w.room = 64;
     }
 
     // SENTINEL: symbol smax may occur, whose upper bound is 2^16 and not the table's last

@@ -175,7 +175,10 @@ struct RangeEncoder {
 
         const int n1 = __builtin_clz(low ^ high);       // low < high always
         // the n1 agreed bits (none if n1 = 0) with the pending complements after the first
-        const uint32_t pe = n1 > 0 ? pend : 0u;
+        // n1 - 1 is needed below; computed as n1 + 0xFFFFFFFF its carry says whether n1 > 0
+        uint32_t n1m1;
+        const bool agreed = __builtin_uadd_overflow((uint32_t)n1, 0xFFFFFFFFu, &n1m1);
+        const uint32_t pe = agreed ? pend : 0u;
         const int m = n1 + (int)pe;
         if (__builtin_expect(m > 32, 0)) {
             const uint32_t bits = low >> ((32 - n1) & 31);
@@ -185,7 +188,7 @@ struct RangeEncoder {
             const uint32_t bits = __builtin_amdgcn_ubfe(low, (uint32_t)(32 - n1), (uint32_t)n1);
             // ((1 << pe) - 1) << (n1 - 1), pe <= 31 here; with n1 = 0, pe is 0 and so is the mask
             uint32_t fill;
-            asm("v_bfm_b32 %0, %1, %2" : "=v"(fill) : "v"(pe), "v"(n1 - 1));
+            asm("v_bfm_b32 %0, %1, %2" : "=v"(fill) : "v"(pe), "v"(n1m1));
             w.template put<FIRST>(bits + fill, m);
         }
         // E3 run: leading zeros of (~low | high) below the first differing bit

@@ -97,6 +97,15 @@ __device__ __forceinline__ uint32_t store16f(float f)
     return DT == CG_DT_BF16 ? float_to_bf16_bits(f) : float_to_f16_bits(f);
 }
 
+// (x + x) << n, i.e. x << (n + 1), in one instruction (n + 1 may be 32: the result is then 0
+// if the bit shifted out last is the only one left, which a plain shift by n + 1 cannot express)
+__device__ __forceinline__ uint32_t shift_left_one_more(uint32_t x, int n)
+{
+    uint32_t r;
+    asm("v_add_lshl_u32 %0, %1, %1, %2" : "=v"(r) : "v"(x), "v"(n));
+    return r;
+}
+
 // 24-bit multiply, low 32 bits of the product, as an unsigned value (HIP's __umul24 returns
 // int, which would turn a following >> into an arithmetic shift).
 __device__ __forceinline__ uint32_t mul24(uint32_t a, uint32_t b) { return (uint32_t)__umul24(a, b); }

@@ -304,7 +304,7 @@ __device__ __forceinline__ void decode_symbol(const DecodeArgs &a, DecodeLane &s
     // E3 run: positions below the first differing bit where low has 1 and high has 0, i.e.
     // leading zeros of (~low | high) once that bit is shifted out; the run always ends
     // inside the word because the interval is wider than one
-    const uint32_t z = ((s.low & high) | (~s.low & 0xFFFFFFFFu)) << ((n1 + 1) & 31);   // one bit-field insert
+    const uint32_t z = shift_left_one_more((s.low & high) | (~s.low & 0xFFFFFFFFu), n1);
     const int n = n1 + __builtin_clz(z);
     // bit 31 of low would be cleared here (the underflow steps subtract a quarter); it is left
     // as it falls: low and high = low + width - 1 then carry the same extra 2^31 modulo 2^32,

@@ -192,7 +192,7 @@ struct RangeEncoder {
             w.template put<FIRST>(bits + fill, m);
         }
         // E3 run: leading zeros of (~low | high) below the first differing bit
-        const uint32_t z = ((low & high) | ~low) << ((n1 + 1) & 31);
+        const uint32_t z = shift_left_one_more((low & high) | ~low, n1);
         const int k = __builtin_clz(z);
         const int n = n1 + k;
         pend = pend - pe + (uint32_t)k;

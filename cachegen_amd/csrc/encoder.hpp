@@ -70,8 +70,11 @@ struct BitWriter {
 
     // append the low m bits of v (v < 2^m), 0 <= m <= 32 (m = 0 needs v = 0).  ROOM: the caller
     // knows that at most 32 bits are waiting (it has just called flush_word), so they fit.
+    // `more` (default 0): a second addend, for callers whose value is a sum of two parts that
+    // together stay below 2^m; the freshly shifted accumulator has m zero bits at the bottom, so
+    // the parts are added in (one three-operand add) instead of summed and then or-ed in
     template <bool ROOM = false>
-    __device__ __forceinline__ void put(uint32_t v, int m)
+    __device__ __forceinline__ void put(uint32_t v, int m, uint32_t more = 0)
     {
         uint32_t left;
         if (__builtin_expect(__builtin_usub_overflow(room, (uint32_t)m, &left), 0) && !ROOM) {
@@ -79,7 +82,8 @@ struct BitWriter {
             left = room - (uint32_t)m;
         }
         room = left;
-        acc = (acc << m) | v;
+        acc <<= m;
+        acc = (acc & 0xFFFFFFFF00000000ull) | (uint32_t)((uint32_t)acc + v + more);
     }
 
     // one bit, then `count` copies of its complement (any count): the general form of
@@ -189,7 +193,7 @@ struct RangeEncoder {
             // ((1 << pe) - 1) << (n1 - 1), pe <= 31 here; with n1 = 0, pe is 0 and so is the mask
             uint32_t fill;
             asm("v_bfm_b32 %0, %1, %2" : "=v"(fill) : "v"(pe), "v"(n1m1));
-            w.template put<FIRST>(bits + fill, m);
+            w.template put<FIRST>(bits, m, fill);
         }
         // E3 run: leading zeros of (~low | high) below the first differing bit
         const uint32_t z = shift_left_one_more((low & high) | ~low, n1);

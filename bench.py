@@ -28,7 +28,7 @@ MEASURED_DECODE_TRAFFIC_BYTES = {"config2": 1366.1e6}
 # VALU wave-instructions per launch of decode_streams_kernel (rocprofv3 --pmc SQ_INSTS_VALU, same
 # profile).  The kernel's own limit is the issue of these: one per 4 cycles per SIMD for most
 # of them, 1024 SIMDs, at the clock the profile's GRBM_GUI_ACTIVE gives (2.3 GHz).
-MEASURED_DECODE_VALU_INSTS = {"config2": 387.26e6}
+MEASURED_DECODE_VALU_INSTS = {"config2": 378.91e6}
 VALU_ISSUE_PER_SECOND = 1024 * 2.3e9 / 4
 
 WORKLOADS = {

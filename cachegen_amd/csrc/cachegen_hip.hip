@@ -265,10 +265,12 @@ int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int
         a.sym4 = sym4;
         if (chunk_tokens <= kSub) {
             // one sub-chunk per chunk: the encoder builds the tables itself
-            CG_DISPATCH_BS(block, (encode_streams_kernel<BS, true, true, true, true><<<grid, blk, shmem, s>>>(a)));
+            if (fused_scan) encode_streams_kernel<kSlotTile, true, true, true, true, true><<<grid, blk, shmem, s>>>(a);
+            else CG_DISPATCH_BS(block, (encode_streams_kernel<BS, true, true, true, true><<<grid, blk, shmem, s>>>(a)));
         } else {
             if (int rc = launch_cdf(nullptr, sym4, nsub, rows, T, C, 0, 0, 0, max_bins, chunk_tokens, tables, s)) return rc;
-            CG_DISPATCH_BS(block, (encode_streams_kernel<BS, true, true, false, true><<<grid, blk, shmem, s>>>(a)));
+            if (fused_scan) encode_streams_kernel<kSlotTile, true, true, false, true, true><<<grid, blk, shmem, s>>>(a);
+            else CG_DISPATCH_BS(block, (encode_streams_kernel<BS, true, true, false, true><<<grid, blk, shmem, s>>>(a)));
         }
     } else {
         // any shape or alignment: byte symbols [2L, T, C]

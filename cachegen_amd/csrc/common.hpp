@@ -119,6 +119,10 @@ __device__ __forceinline__ uint32_t scale_span(uint32_t sh, uint32_t sl, uint32_
     return mul24(sh, c) + (mul24(sl, c) >> 16);
 }
 
+// Fourth word of a buffer descriptor for raw (untyped, unswizzled) access on gfx9-family
+// GPUs: 32-bit data format, everything else off.
+constexpr int kBufferWord3 = 0x00020000;
+
 // Pointers into LDS, for loads with immediate offsets.
 typedef __attribute__((address_space(3))) const uint16_t lds_u16;
 typedef __attribute__((address_space(3))) const float lds_f32;

@@ -32,10 +32,6 @@ namespace {
 // the final interval for every continuation, so the n symbols that were encoded decode
 // identically.  Word loads past the last word of the byte buffer return zeros.
 
-// Fourth word of a buffer descriptor for raw (untyped, unswizzled) access on gfx9-family
-// GPUs: 32-bit data format, everything else off.
-constexpr int kBufferWord3 = 0x00020000;
-
 // The most bits one symbol can move for a table without zero-width entries.
 constexpr uint32_t kSymbolBits = 18;
 

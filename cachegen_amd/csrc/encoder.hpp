@@ -23,12 +23,20 @@ namespace {
 // of positions below those where low has ones and high has zeros.  One combined shift by
 // n = n1 + k renormalises low and high; n <= 18 for any table whose symbols all have
 // non-zero width, because the span stays above 2^30 between symbols.
-template <bool ALIGNED>
+constexpr int kSlotTile = 256;      // streams per tile of the encoder's scratch
+
+// TILE: the stream's words go to a tile of the scratch (word w of the tile's stream t at the
+// tile's word w * kSlotTile + t) through a buffer descriptor that covers exactly the tile: a
+// word or byte past the stream's capacity falls outside the descriptor and is dropped by the
+// hardware, so nothing is compared or counted per word.
+template <bool ALIGNED, bool TILE = false>
 struct BitWriter {
     uint8_t *wptr;          // where the next word goes
     int wstride;            // bytes from one word of the stream to the next (4: contiguous)
     int cap;
     int nbytes;
+    __amdgpu_buffer_rsrc_t tile;    // TILE: the block's tile
+    uint32_t voff, voff0;           // TILE: byte offset in the tile of the next word, and of the first
     uint64_t acc;           // the low 64 - room bits are waiting to be written; bits above are stale
     // free bits of the accumulator: counted this way, the subtraction that books a put borrows
     // exactly when the bits do not fit, and that borrow is the test
@@ -43,6 +51,11 @@ struct BitWriter {
 
     __device__ __forceinline__ void store_word(uint32_t word)
     {
+        if (TILE) {
+            __builtin_amdgcn_raw_buffer_store_b32((int)__builtin_bswap32(word), tile, (int)voff, 0, 0);
+            voff += kSlotTile * 4;
+            return;
+        }
         if (__builtin_expect(nbytes + 4 <= cap, 1)) {
             if (ALIGNED) {
                 *reinterpret_cast<uint32_t *>(wptr) = __builtin_bswap32(word);
@@ -109,10 +122,12 @@ struct BitWriter {
         flush_word();
         flush_word();
         const int nacc = 64 - (int)room;
+        if (TILE) nbytes = (int)((voff - voff0) / kSlotTile);     // four bytes per word written
         if (nacc > 0) {
             uint32_t r = (uint32_t)(acc << (32 - nacc));
             for (int left = nacc, j = 0; left > 0; left -= 8, ++j) {
-                if (nbytes < cap) wptr[j] = (uint8_t)(r >> 24);
+                if (TILE) __builtin_amdgcn_raw_buffer_store_b8((char)(r >> 24), tile, (int)(voff + j), 0, 0);
+                else if (nbytes < cap) wptr[j] = (uint8_t)(r >> 24);
                 nbytes++;
                 r <<= 8;
             }
@@ -125,7 +140,7 @@ struct BitWriter {
 // the full range 2^32 (the initial state, and any later interval that is exactly a binary
 // fraction), where floor(span * c / 2^16) is simply c << 16.  Renormalising by n bits maps
 // span to span << n for E1/E2 and E3 steps alike.
-template <int BS, bool ALIGNED>
+template <int BS, bool ALIGNED, bool TILE = false>
 struct RangeEncoder {
     lds_char *col;          // this lane's table column: entry e at byte e * 2 * TableStride<BS>::k16
     uint32_t smax;          // lp - 2: the largest symbol
@@ -133,7 +148,7 @@ struct RangeEncoder {
     // the coded symbol's two table entries, each shifted left by 16: only ever written by
     // loads into the upper half, so that the lower halves stay zero
     uint32_t bound_lo, bound_hi;
-    BitWriter<ALIGNED> w;
+    BitWriter<ALIGNED, TILE> w;
 
     __device__ __forceinline__ void init(const uint16_t *column, int lp, uint8_t *dst, int wstride, int cap)
     {
@@ -148,6 +163,7 @@ struct RangeEncoder {
         w.wstride = wstride;
         w.cap = cap;
         w.nbytes = 0;
+        w.voff = w.voff0 = 0;
         w.acc = 0;
         w.room = 64;
     }
@@ -230,7 +246,6 @@ struct EncodeArgs {
     StreamGrid sg;
 };
 
-constexpr int kSlotTile = 256;      // streams per tile of the encoder's scratch
 
 template <bool B>
 struct BoolTag {
@@ -240,7 +255,7 @@ struct BoolTag {
 // PACKED: symbols come from sym4.  FUSE_CDF (PACKED only, one sub-chunk per chunk): the
 // block first builds its own tables from the same words and writes them out.
 // SLOTS: stream g of the launch is written to out[g * cap ...] (the fused path's scratch).
-template <int BS, bool ALIGNED, bool PACKED, bool FUSE_CDF, bool SLOTS>
+template <int BS, bool ALIGNED, bool PACKED, bool FUSE_CDF, bool SLOTS, bool TILE = false>
 __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
 {
     extern __shared__ uint16_t tab[];
@@ -297,12 +312,19 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
     }
     if (!id.active) return;
 
-    RangeEncoder<BS, ALIGNED> enc;
+    RangeEncoder<BS, ALIGNED, TILE> enc;
     const int64_t stream = (id.sub * a.sg.rows + id.row) * a.sg.nc + id.ch;
     // SLOTS: the scratch is cut into tiles of kSlotTile streams; word w of a tile's stream t is
     // the tile's word w * kSlotTile + t, so that the words the lanes of a wavefront write, and
     // the words the compaction reads, lie side by side
-    if (SLOTS)
+    if (TILE) {
+        // the block is exactly one tile (the host launches this form only then): blockIdx.x is
+        // the tile, tid the stream's place in it
+        enc.init(col, lp, nullptr, 0, a.cap);
+        enc.w.tile = __builtin_amdgcn_make_buffer_rsrc((void *)(a.out + (int64_t)blockIdx.x * ((int64_t)kSlotTile * a.cap)), 0,
+                                                       kSlotTile * a.cap, kBufferWord3);
+        enc.w.voff = enc.w.voff0 = (uint32_t)tid * 4u;
+    } else if (SLOTS)
         enc.init(col, lp, a.out + (stream / kSlotTile) * ((int64_t)kSlotTile * a.cap) + (stream % kSlotTile) * 4,
                  kSlotTile * 4, a.cap);
     else

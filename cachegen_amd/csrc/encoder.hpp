@@ -265,19 +265,33 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
     const int64_t ch0 = id.ch - tid;
     uint16_t *col = tab + tid;
     uint16_t *cdf_block = a.cdf + ((id.chunk * a.sg.rows + id.row) * a.sg.nc + ch0) * lp;
-    const uint32_t *wp = nullptr;
     const int nwords = (id.n + 3) >> 2;
-    if (PACKED) wp = a.sym4 + ((id.row * a.nsub + id.sub) * kWordsPerSub) * a.sg.nc + id.ch;
+    // PACKED: the sub-chunk's words ([word][channel]) are read through a buffer descriptor that
+    // ends with its last word row: the lane's channel is the vector offset, the word row the
+    // scalar one, and a row past the end (or the offset of a lane without a channel) reads
+    // zero, so a load costs no address arithmetic, compare or branch.
+    __amdgpu_buffer_rsrc_t symbols_rsrc;
+    uint32_t symbols_voff = 0xFFFFFFFCu;
+    const uint32_t row_bytes = (uint32_t)a.sg.nc * 4u;
+    if (PACKED) {
+        const int64_t first = ((id.row * a.nsub + id.sub) * kWordsPerSub) * a.sg.nc;        // uniform over the block
+        const uint32_t lo32 = __builtin_amdgcn_readfirstlane((uint32_t)first);
+        const uint32_t hi32 = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)first >> 32));
+        symbols_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(a.sym4 + (int64_t)(((uint64_t)hi32 << 32) | lo32)), 0,
+                                                         (int)((uint32_t)nwords * row_bytes), kBufferWord3);
+        if (id.active) symbols_voff = (uint32_t)id.ch * 4u;
+    }
 
-    // PACKED: half a sub-chunk (32 words = 128 symbols) at a time is loaded into registers
-    // and indexed by the (uniform) loop counter, so the coding loop has no loads to wait
-    // for and its stores never hold it up.
+    // Half a sub-chunk (32 words = 128 symbols) at a time is loaded into registers and indexed
+    // by the (uniform) loop counter, so the coding loop has no loads to wait for and its stores
+    // never hold it up.
     typedef uint32_t words32 __attribute__((ext_vector_type(32)));
     words32 words;
     auto load_half = [&](int h) {
 #pragma unroll
         for (int w = 0; w < 32; ++w)
-            words[w] = (id.active && h * 32 + w < nwords) ? wp[(int64_t)(h * 32 + w) * a.sg.nc] : 0u;
+            words[w] = __builtin_amdgcn_raw_buffer_load_b32(symbols_rsrc, (int)symbols_voff,
+                                                            (int)((uint32_t)(h * 32 + w) * row_bytes), 0);
     };
 
     if (FUSE_CDF) {

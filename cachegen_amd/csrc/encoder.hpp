@@ -304,7 +304,8 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
             const uint32_t one = (tid & 1) ? 0x10000u : 1u;
             for (int h = 0; h * 32 < nwords; ++h) {
                 load_half(h);
-                const int wn = nwords - h * 32 < 32 ? nwords - h * 32 : 32;
+                // uniform; kept in a scalar register so that the loop test is scalar too
+                const int wn = __builtin_amdgcn_readfirstlane(nwords - h * 32 < 32 ? nwords - h * 32 : 32);
 #pragma unroll 1
                 for (int w = 0; w < wn; ++w) {
                     const uint32_t v = words[w];
@@ -359,7 +360,8 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
         if (PACKED) {
             for (int h = 0; h * 32 < nwords; ++h) {
                 load_half(h);
-                const int wn = nwords - h * 32 < 32 ? nwords - h * 32 : 32;
+                // uniform; kept in a scalar register so that the loop test is scalar too
+                const int wn = __builtin_amdgcn_readfirstlane(nwords - h * 32 < 32 ? nwords - h * 32 : 32);
 #pragma unroll 1
                 for (int w = 0; w < wn; ++w) {
                     const uint32_t v = words[w];

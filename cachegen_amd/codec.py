@@ -149,6 +149,23 @@ def encode_kv(kv, key_bins, value_bins, chunk_tokens=None, fmt="vllm", max_bins=
             status=torch.empty(1, dtype=torch.int32, device=dev),
             num_layers=L, num_tokens=T, num_heads=H, head_size=D, chunk_tokens=S, max_bins=max_bins,
             delta_group=int(delta_group))
+    else:
+        # a reused result must have been made for this geometry: the kernels write every field
+        want = {"cdf": (nchunks, 2 * L, C, max_bins + 1), "maxima": (2, L, T), "lengths": (nsub, 2 * L, C),
+                "offsets": (nstreams + 1,), "status": (1,)}
+        for name, shape in want.items():
+            t = getattr(out, name)
+            if tuple(t.shape) != shape or not t.is_contiguous() or t.device != dev:
+                raise RuntimeError("encode_kv: `out.%s` has shape %s, this call needs %s (contiguous, on %s)"
+                                   % (name, tuple(t.shape), shape, dev))
+        if out.maxima.dtype != kv.dtype or out.cdf.dtype != torch.int16 or out.lengths.dtype != torch.int32 \
+                or out.offsets.dtype != torch.int64 or out.payload.dtype != torch.uint8 or out.status.dtype != torch.int32:
+            raise RuntimeError("encode_kv: `out` holds tensors of the wrong dtype for this call")
+        if not out.payload.is_contiguous() or out.payload.device != dev:
+            raise RuntimeError("encode_kv: `out.payload` must be a contiguous tensor on %s" % dev)
+        if (out.num_layers, out.num_tokens, out.num_heads, out.head_size, out.chunk_tokens, out.max_bins,
+                out.delta_group) != (L, T, H, D, S, max_bins, int(delta_group)):
+            raise RuntimeError("encode_kv: `out` was made for another geometry")
     with torch.cuda.device(dev):
         _lib.check(lib.cg_encode_kv(
             kv.data_ptr(), _DT[kv.dtype], L, T, H, D, sl, skv, st, sh,
@@ -191,6 +208,28 @@ def decode_kv(cdf, maxima, offsets, payload, key_bins, value_bins, num_layers, n
     maxima = maxima.contiguous()
     if maxima.dtype not in _DT:
         raise RuntimeError("row maxima must be float16 or bfloat16")
+    # the kernel indexes every input by the geometry: refuse inputs that do not have it
+    S = int(chunk_tokens)
+    if S <= 0:
+        raise RuntimeError("chunk_tokens must be positive")
+    C = H * D
+    nchunks, nsub = -(-T // S), num_subchunks(T, S)
+    if key_bins.numel() != L or value_bins.numel() != L:
+        raise RuntimeError("bins vectors must have one entry per layer (%d), got %d and %d"
+                           % (L, key_bins.numel(), value_bins.numel()))
+    if cdf.dim() != 4 or tuple(cdf.shape[:3]) != (nchunks, 2 * L, C) or cdf.dtype != torch.int16:
+        raise RuntimeError("tables must be int16 [%d, %d, %d, Lp], got %s %s"
+                           % (nchunks, 2 * L, C, cdf.dtype, tuple(cdf.shape)))
+    if tuple(maxima.shape) != (2, L, T):
+        raise RuntimeError("row maxima must have shape (2, %d, %d), got %s" % (L, T, tuple(maxima.shape)))
+    if offsets.dtype != torch.int64 or offsets.numel() != nsub * 2 * L * C + 1 or not offsets.is_contiguous():
+        raise RuntimeError("offsets must be a contiguous int64 tensor of %d entries, got %s of %d"
+                           % (nsub * 2 * L * C + 1, offsets.dtype, offsets.numel()))
+    if payload.dtype != torch.uint8 or not payload.is_contiguous() or payload.numel() == 0:
+        raise RuntimeError("payload must be a contiguous, non-empty uint8 tensor")
+    for name, t in (("maxima", maxima), ("offsets", offsets), ("payload", payload)):
+        if t.device != dev:
+            raise RuntimeError("%s is on %s, the tables on %s" % (name, t.device, dev))
     key_bins = key_bins.to(device=dev, dtype=torch.float32).contiguous()
     value_bins = value_bins.to(device=dev, dtype=torch.float32).contiguous()
     with torch.cuda.device(dev):

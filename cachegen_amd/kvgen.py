@@ -9,8 +9,6 @@ the token axis every channel is an AR(1) process with correlation `rho`:
 The result is cast to 16 bits and laid out [L, 2, T, H, D] ("vllm" layout of
 LMCache/lmcache/storage_backend/serde/cachegen_encoder.py:341-346).
 """
-import math
-
 import torch
 
 
@@ -56,4 +54,4 @@ def entropy_bits(symbols, nbins):
     return float(-(p * torch.log2(p)).sum())
 
 
-__all__ = ["make_kv", "kv_nbytes", "entropy_bits", "math"]
+__all__ = ["make_kv", "kv_nbytes", "entropy_bits"]

@@ -108,7 +108,8 @@ class CacheGenDeserializer(Deserializer):
         if h["num_layers"] != self.key_bins.numel():
             raise ValueError("blob has %d layers, this deserializer's model %d"
                              % (h["num_layers"], self.key_bins.numel()))
-        offsets = codec.scan_lengths(lengths)
+        # a stream occupies min(length, 256) bytes of the payload (wire.py checks the same sum)
+        offsets = codec.scan_lengths(lengths.clamp(max=wire.MAX_STREAM_BYTES))
         result = codec.decode_kv(cdf, maxima, offsets, payload, self.key_bins, self.value_bins,
                                  h["num_layers"], h["num_tokens"], h["num_heads"], h["head_size"],
                                  chunk_tokens=h["chunk_tokens"], fmt=self.fmt, delta_group=h["delta_group"],

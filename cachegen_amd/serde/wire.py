@@ -474,7 +474,9 @@ def unpack_to_device(blob, device, defer_checks=False):
     off, size = geo["lengths"]
     host_lengths = np.frombuffer(blob, dtype=np.uint16 if h["lengths_u16"] else np.int32, count=h["nsub"] * 2 * L * C,
                                  offset=off)
-    if int(host_lengths.sum(dtype=np.int64)) != h["payload_bytes"] or (host_lengths.size and int(host_lengths.min()) < 0):
+    # one rule everywhere: a stream occupies min(length, 256) bytes of the payload
+    if int(np.minimum(host_lengths, MAX_STREAM_BYTES).sum(dtype=np.int64)) != h["payload_bytes"] \
+            or (host_lengths.size and int(host_lengths.min()) < 0):
         raise ValueError("wire container: payload size is not the sum of the stream lengths")
     h["check"] = lambda: None
 

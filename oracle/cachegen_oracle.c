@@ -107,7 +107,7 @@ static uint16_t store16(float f, int dt)
 /* Quantization: torch_quant_vectorized, encoder.py:42-59.                   */
 /*   MAX    = bins // 2 - 1                      (float32 per layer)         */
 /*   max1   = amax(|x|) over the channels of one (layer, token) row, kept in */
-/*            the input's 16-bit dtype                                       */
+/*            the input's 16-bit dtype (a row with NaNs: see below)          */
 /*   factor = MAX / max1                         (float32 divide)            */
 /*   sym    = round_half_even(x * factor + MAX)  (float32 mul, then add)     */
 /*            cast to int8.  A NaN (all-zero row: 0 * inf) casts to 0.       */
@@ -122,15 +122,19 @@ void cgo_quantize(const uint16_t *x, int dt, int64_t nl, int64_t nt, int64_t nc,
         for (int64_t t = 0; t < nt; t++) {
             const uint16_t *row = x + l * sl + t * st;
             const float maxq = floorf(bins[l] / 2.0f) - 1.0f;
+            /* |x| of a 16-bit float is its bit pattern without the sign, and for patterns
+             * that are not NaN the order of the patterns as integers is the order of the
+             * values, so amax(|x|) is the largest sign-stripped pattern.  A NaN in the row
+             * makes amax NaN (torch propagates it) without saying which payload survives
+             * when the row holds several: the rule here is the largest pattern, which is
+             * a NaN whenever the row has one (every NaN pattern is above infinity's). */
             uint16_t mbits = 0;
-            float mval = 0.0f;
-            int have_nan = 0;
             for (int64_t c = 0; c < nc; c++) {
-                float a = fabsf(load16(row + c, dt));
-                if (a != a) { if (!have_nan) { have_nan = 1; mbits = row[c] & 0x7FFFu; mval = a; } }
-                else if (!have_nan && (c == 0 || a > mval)) { mval = a; mbits = row[c] & 0x7FFFu; }
+                const uint16_t a = row[c] & 0x7FFFu;
+                if (a > mbits) mbits = a;
             }
             max_out[l * nt + t] = mbits;
+            const float mval = load16(&mbits, dt);
             const float factor = maxq / mval;
             uint8_t *out = sym + (l * nt + t) * nc;
             for (int64_t c = 0; c < nc; c++) {

@@ -48,6 +48,17 @@ KNOWN_ANSWERS = {
         {"cdf": [0, 16384, 49152, 65535], "symbols": [1, 2], "bytes": [0xA8]},   # pending, 10 1 | 01
         {"cdf": [0, 16384, 49152, 65535], "symbols": [1] * 40,
          "bytes": list(int("0" + "1" * 41 + "000000", 2).to_bytes(6, "big"))},    # 40 pending: 0 then 41 ones
+        # a table that is not dyadic, so that span * c is not a multiple of 2^16 and the floor of
+        # `(span * c) >> 16` matters (worked through step by step in tests/test_oracle_pins.py:
+        # rounding to nearest instead of truncating gives the five bytes 00 07 00 30 ff)
+        {"cdf": [0, 7, 65535], "symbols": [1, 0, 1, 0, 0], "bytes": [0x00, 0x07, 0x00, 0x30, 0xFF, 0x00]},
+    ],
+    "decoder_boundary": [
+        # hand-built streams (not encoder output) whose code value sits exactly on, and one below,
+        # a symbol boundary low + floor(span * c / 2^16) with a dropped fraction above one half:
+        # 12 zero bits, then the 32-bit value, zero fill
+        {"cdf": [0, 7, 65535], "bytes": [0x00, 0x07, 0x00, 0x30, 0xFE, 0xA0], "symbols": [1, 0, 1]},   # value 0x70030FEA
+        {"cdf": [0, 7, 65535], "bytes": [0x00, 0x07, 0x00, 0x30, 0xFE, 0x90], "symbols": [1, 0, 0]},   # value 0x70030FE9
     ],
     "dequantize": [
         # ((s - C) / C) * max in float32, then nearest-even to float16; C = bins//2 - 1

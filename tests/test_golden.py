@@ -30,6 +30,8 @@ def test_oracle_known_answers(oracle):
         data, n = oracle.encode_stream(k["cdf"], k["symbols"])
         assert list(data) == k["bytes"] and n == len(k["bytes"])
         assert oracle.decode_stream(k["cdf"], bytes(k["bytes"]), len(k["symbols"])).tolist() == k["symbols"]
+    for k in KA["decoder_boundary"]:
+        assert oracle.decode_stream(k["cdf"], bytes(k["bytes"]), len(k["symbols"])).tolist() == k["symbols"]
     for k in KA["dequantize"]:
         out = oracle.dequantize(np.array([[k["symbols"]]], dtype=np.uint8), [float(k["bins"])],
                                 np.array([[k["max"]]], dtype=np.float16).view(np.uint16))
@@ -73,6 +75,19 @@ def test_hip_known_answers():
             back = torch.zeros((1, len(k["symbols"]), 1), dtype=torch.uint8, device=DEV)
             tac.decode_fast_new(cdf, out, lens, back)
             assert back.flatten().tolist() == k["symbols"]
+    for k in KA["decoder_boundary"]:
+        cdf = torch.tensor(np.array(k["cdf"], dtype=np.uint16).view(np.int16), device=DEV).view(1, 1, -1)
+        n = len(k["symbols"])
+        data = torch.tensor(k["bytes"], dtype=torch.uint8, device=DEV)
+        back = torch.zeros((1, n, 1), dtype=torch.uint8, device=DEV)
+        prefix = torch.tensor([[len(k["bytes"])]], dtype=torch.int64, device=DEV)
+        tac.decode_fast_prefsum(cdf, data, prefix, back)
+        assert back.flatten().tolist() == k["symbols"]
+        padded = torch.zeros((1, 1, 256), dtype=torch.uint8, device=DEV)
+        padded[0, 0, :len(k["bytes"])] = data
+        back2 = torch.zeros((1, n, 1), dtype=torch.uint8, device=DEV)
+        tac.decode_fast_new(cdf, padded, torch.tensor([[len(k["bytes"])]], dtype=torch.int32, device=DEV), back2)
+        assert back2.flatten().tolist() == k["symbols"]
 
 
 @pytest.mark.gpu

@@ -169,6 +169,31 @@ def test_nan_and_infinite_rows_match_oracle(oracle):
             assert nan_ref.any() and np.array_equal(got[~nan_ref], ref[~nan_ref]), (dtype, out_dtype)
 
 
+def test_rows_with_several_different_nans_keep_the_largest_pattern(oracle):
+    """Two or three NaNs with different payloads and signs in one row: the stored row maximum
+    is the largest sign-stripped bit pattern in the fused path, in the plain quantiser and in
+    the oracle alike."""
+    codec, _ = _mods()
+    L, T, H, D = 1, 8, 2, 64
+    for dtype, dt, pats in ((torch.float16, 0, [0x7E01, 0xFE55, 0x7C01]), (torch.bfloat16, 1, [0x7FC1, 0xFFD5, 0x7F81])):
+        g = torch.Generator().manual_seed(17)
+        raw = torch.randn((L, 2, T, H * D), generator=g).to(dtype).view(torch.int16).numpy().view(np.uint16).copy()
+        raw[0, 0, 2, 100], raw[0, 0, 2, 3], raw[0, 0, 2, 77] = pats            # the largest one in the middle
+        raw[0, 1, 5, 9], raw[0, 1, 5, 120] = pats[2], pats[0]
+        x = torch.from_numpy(raw.view(np.int16)).view(dtype).reshape(L, 2, T, H, D)
+        bins = torch.tensor([32.0])
+        enc = codec.encode_kv(x.to(DEV), bins, bins, chunk_tokens=T)
+        enc.check()
+        want = oracle.encode_function(raw, bins.numpy(), bins.numpy(), dt)
+        got_max = enc.maxima.cpu().view(torch.int16).numpy().view(np.uint16)
+        assert got_max[0, 0, 2] == (pats[1] & 0x7FFF) and got_max[1, 0, 5] == pats[0]
+        assert np.array_equal(got_max[0], want["max_tensors_key"]) and np.array_equal(got_max[1], want["max_tensors_value"])
+        assert np.array_equal(enc.cdf[0].cpu().numpy().view(np.uint16), want["cdf"])
+        assert np.array_equal(enc.payload[:enc.total_bytes()].cpu().numpy(), want["data_chunks"][0][0])
+        sym, maxima = codec.quantize_kv(x.to(DEV), bins.to(DEV), bins.to(DEV))
+        assert np.array_equal(maxima.cpu().view(torch.int16).numpy().view(np.uint16), got_max)
+
+
 @pytest.mark.parametrize("nt", [1, 2, 7])
 def test_streams_that_begin_in_the_last_word_of_an_exact_size_buffer(oracle, nt):
     """The byte buffer ends with the last stream, and that stream is so short that it starts

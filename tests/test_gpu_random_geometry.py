@@ -16,11 +16,18 @@ def bits(t):
     return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
 
 
-def draw_case(rng):
+def draw_case(rng, wide=False):
     L = int(rng.integers(1, 5))
     H = int(rng.choice([1, 2, 3, 4, 8]))
     D = int(rng.choice([8, 16, 20, 32, 40, 64, 128]))
     T = int(rng.integers(1, 900))
+    if wide:
+        # 1280 to 4096 channels: the fused quantiser's four and eight loads per lane, many
+        # channel tiles per row, a partial last tile (1280 = 5 x 256, 3072 = 12 x 256 are whole;
+        # 24 x 72 = 1728 is not)
+        L = int(rng.integers(1, 4))
+        H, D = [(16, 128), (32, 128), (32, 64), (24, 72), (10, 128), (24, 128)][int(rng.integers(0, 6))]
+        T = int(rng.integers(1, 600))
     S = int(rng.choice([T, 256, int(rng.integers(1, T + 1)), 300, 512]))
     top = int(rng.choice(LEVELS))
     lower = [b for b in LEVELS if b <= top]
@@ -36,11 +43,20 @@ def draw_case(rng):
 
 @pytest.mark.parametrize("seed", range(12))
 def test_random_case_matches_oracle(oracle, seed):
+    run_cases(oracle, seed, 4, False)
+
+
+@pytest.mark.parametrize("seed", range(100, 106))
+def test_random_wide_case_matches_oracle(oracle, seed):
+    run_cases(oracle, seed, 2, True)
+
+
+def run_cases(oracle, seed, ncases, wide):
     from cachegen_amd import codec
     from cachegen_amd.kvgen import make_kv
     rng = np.random.default_rng(9000 + seed)
-    for _ in range(4):
-        L, T, H, D, S, kb, vb, dtype, fmt, kind = draw_case(rng)
+    for _ in range(ncases):
+        L, T, H, D, S, kb, vb, dtype, fmt, kind = draw_case(rng, wide)
         label = dict(L=L, T=T, H=H, D=D, S=S, kb=kb.tolist(), vb=vb.tolist(), dtype=str(dtype), fmt=fmt, kind=kind)
         print(label, flush=True)
         gen = torch.Generator().manual_seed(seed * 100 + T)

@@ -125,3 +125,35 @@ def test_product_code_never_touches_the_oracle():
             if name.endswith((".py", ".hip", ".hpp", ".h")):
                 text = open(os.path.join(folder, name)).read()
                 assert "oracle" not in text.replace("no reference to be at parity", ""), os.path.join(folder, name)
+
+
+def test_decode_kv_refuses_inputs_that_do_not_have_the_geometry():
+    """A blob made for a model with more layers than the bins vectors, or tensors of the wrong
+    shape, is refused on the host before any kernel could index past a buffer."""
+    import torch
+    from cachegen_amd import codec
+    L, T, H, D, S = 2, 300, 2, 8, 256
+    C, nsub = H * D, 2
+    cdf = torch.zeros((2, 2 * L, C, 33), dtype=torch.int16)
+    maxima = torch.zeros((2, L, T), dtype=torch.float16)
+    offsets = torch.zeros(nsub * 2 * L * C + 1, dtype=torch.int64)
+    payload = torch.zeros(64, dtype=torch.uint8)
+    bins = torch.full((L,), 32.0)
+
+    def call(**kw):
+        a = dict(cdf=cdf, maxima=maxima, offsets=offsets, payload=payload, key_bins=bins, value_bins=bins)
+        a.update(kw)
+        return codec.decode_kv(a["cdf"], a["maxima"], a["offsets"], a["payload"], a["key_bins"], a["value_bins"],
+                               L, T, H, D, S, out=torch.empty((L, 2, T, H, D), dtype=torch.float16))
+    with pytest.raises(RuntimeError, match="one entry per layer"):
+        call(key_bins=torch.full((L - 1,), 32.0))
+    with pytest.raises(RuntimeError, match="tables must be"):
+        call(cdf=cdf[:1])
+    with pytest.raises(RuntimeError, match="tables must be"):
+        call(cdf=torch.zeros((2, 2 * L + 2, C, 33), dtype=torch.int16))
+    with pytest.raises(RuntimeError, match="row maxima must have shape"):
+        call(maxima=maxima[:, :, :-1])
+    with pytest.raises(RuntimeError, match="offsets must be"):
+        call(offsets=offsets[:-1])
+    with pytest.raises(RuntimeError, match="payload must be"):
+        call(payload=payload[:0])

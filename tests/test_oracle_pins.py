@@ -81,6 +81,24 @@ def test_quantize_zero_row_gives_zero_symbols(oracle):
     assert mx.view(np.float16).tolist() == [[0.0, 2.0]]
 
 
+def test_quantize_row_maximum_with_several_nans(oracle):
+    """amax(|x|) of a row that holds NaNs is NaN (torch propagates it); which payload is kept
+    when there are several is not specified by torch, so the rule is fixed here: the largest
+    sign-stripped bit pattern.  For rows without NaN that is the ordinary maximum."""
+    for dt, pats, inf in ((0, [0x7E01, 0xFE55, 0x7C01], 0x7C00), (1, [0x7FC1, 0xFFD5, 0x7F81], 0x7F80)):
+        row = np.array([0x3C00, pats[0], 0xBC00, pats[1], pats[2], 0x0000, inf, 0x4000], dtype=np.uint16)
+        sym, mx = oracle.quantize(row.reshape(1, 1, 8), [32.0], dt)
+        assert int(mx[0, 0]) == (pats[1] & 0x7FFF)           # the largest pattern, sign removed
+        assert sym[0, 0].tolist() == [0] * 8                 # every x * (MAX / NaN) is NaN -> 0
+        # torch agrees on what it does specify: the maximum is a NaN
+        t = torch.from_numpy(row.view(np.int16).copy()).view(torch.float16 if dt == 0 else torch.bfloat16)
+        assert bool(torch.isnan(torch.amax(torch.abs(t))))
+    # without NaN: infinity wins, symbols of finite values collapse to MAX, of +-inf to NaN -> 0
+    row = np.array([0x3C00, 0xFC00, 0x4000, 0x0000], dtype=np.uint16)
+    sym, mx = oracle.quantize(row.reshape(1, 1, 4), [32.0], 0)
+    assert int(mx[0, 0]) == 0x7C00 and sym[0, 0].tolist() == [15, 0, 15, 15]
+
+
 def _torch_quant(x, bins):
     """Closed form with torch CPU ops: float32 divide, multiply, add, round half even."""
     maxq = (bins // 2 - 1)[:, None, None]
@@ -186,6 +204,43 @@ def test_coder_hand_known_answers(oracle):
     assert oracle.decode_stream(cdf3, bytes([0xA8]), 2).tolist() == [1, 2]
     # empty stream: only the tail "01"
     assert oracle.encode_stream(cdf, []) == (bytes([0x40]), 1)
+
+
+def test_coder_truncates_the_scaled_bounds_on_a_table_that_is_not_dyadic(oracle):
+    """`(span * c) >> 16` drops the fraction (enc_new.cu:272-273, dec_new.cu:280-281).  With
+    cdf = [0, 7, 65535] the products stop being multiples of 2^16 from the third symbol on;
+    worked by hand for the symbols 1, 0, 1, 0, 0 (symbol 1 is the last one: upper bound 2^16):
+
+      start                 low 00000000  high FFFFFFFF  span 1_0000_0000
+      s=1  T(7)  = 7<<16 = 70000, T(2^16) = span        -> low 00070000 high FFFFFFFF, no bits out
+      s=0  span FFF90000: T(7) = 6FFCF0000>>16 = 6FFCF (exact)
+                                                        -> low 00070000 high 000DFFCE
+           twelve leading bits agree: emits 000000000000 -> low 70000000 high DFFCEFFF
+      s=1  span 6FFCF000: T(7) = 3_0FEA_9000>>16 = 30FEA (drops 0.5625), T(2^16) = 6FFCF000
+                                                        -> low 70030FEA high DFFCEFFF, no bits out
+      s=0  span 6FF9E016: T(7) = 3_0FD5_209A>>16 = 30FD5 (drops 0.127)
+                                                        -> low 70030FEA high 70061FBE
+           thirteen bits agree: emits 0111000000000     -> low 61FD4000 high C3F7DFFF
+      s=0  span 61FAA000: T(7) = 2_ADDA_6000>>16 = 2ADDA (drops 0.375)
+                                                        -> low 61FD4000 high 61FFEDD9
+           fourteen bits agree: emits 01100001111111    -> low 50000000 high FB767FFF
+      end  low >= 2^30: emits 1, then the pending count (0 + 1) of zeros: 10
+
+    41 bits: 000000000000 0111000000000 01100001111111 10, padded to 00 07 00 30 ff 00.
+    Rounding the third symbol's 30FEA.9 up to 30FEB instead moves low, and the stream then
+    comes out as the five bytes 00 07 00 30 ff."""
+    cdf = [0, 7, 65535]
+    want = bytes([0x00, 0x07, 0x00, 0x30, 0xFF, 0x00])
+    assert oracle.encode_stream(cdf, [1, 0, 1, 0, 0]) == (want, 6)
+    assert oracle.decode_stream(cdf, want, 5).tolist() == [1, 0, 1, 0, 0]
+    # the decoder's side of the same floor, on streams built by hand: after the symbols 1, 0
+    # twelve bits are used up and the state is low 70000000, span 6FFCF000, so the boundary
+    # between symbols 0 and 1 is the code value 70000000 + 30FEA (30FEB if it were rounded)
+    on_it = (0x70030FEA << 4).to_bytes(6, "big")         # 12 zero bits, the value, 4 zero bits
+    below = (0x70030FE9 << 4).to_bytes(6, "big")
+    assert on_it == bytes([0x00, 0x07, 0x00, 0x30, 0xFE, 0xA0])
+    assert oracle.decode_stream(cdf, on_it, 3).tolist() == [1, 0, 1]
+    assert oracle.decode_stream(cdf, below, 3).tolist() == [1, 0, 0]
 
 
 def test_coder_long_pending_run(oracle):

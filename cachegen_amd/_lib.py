@@ -34,6 +34,7 @@ SIGNATURES = {
                             _P, _P, _P, _P, _P, _I64, _P, _P, _SZ, _P]),
     "cg_scan_workspace": (_SZ, [_I64]),
     "cg_scan_lengths": (_INT, [_P, _I64, _P, _P, _SZ, _P]),
+    "cg_scan_lengths_static": (_INT, [_P, _I64, _P, _P]),
     "cg_tables_to_counts": (_INT, [_P, _INT, _I64, _I64, _P, _P, _P, _P, _P]),
     "cg_pack_counts": (_INT, [_P, _INT, _I64, _I64, _P, _P, _P, _P]),
     "cg_counts_to_tables": (_INT, [_P, _I64, _INT, _I64, _I64, _P, _P, _P, _P, _P, _P]),

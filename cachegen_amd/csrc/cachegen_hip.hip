@@ -20,6 +20,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 
 #include "cachegen_hip.h"
 
@@ -38,12 +39,50 @@
 #include "tables_wire.hpp"
 
 // ======================================================================================
+// Scratch of the entry point that allocates nothing (cg_scan_lengths_static): the partial sums
+// of the multi-block running sum, one int64 per 2048 lengths plus one.  Every GPU the library
+// runs on holds its own copy of this array, at its own address, until the process ends.  In host
+// code the array's name is only a handle for hipGetSymbolAddress: kernels and copies get the
+// device address looked up once per device below, never the name.
+// ======================================================================================
+constexpr int64_t kStaticScanMaxLengths = CG_SCAN_STATIC_MAX_LENGTHS;
+constexpr size_t kStaticScanBytes = (size_t)(kStaticScanMaxLengths / kScanTile + 2) * sizeof(int64_t);
+static __device__ __align__(256) unsigned char scratch[kStaticScanBytes];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_static_scratch_mutex;
+void *g_static_scratch[kMaxDevices];          // device address of `scratch` on each GPU, once looked up
+
+// Device address of `scratch` on the current device (looked up on the first call per device).
+int static_scratch(void **ptr)
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(CG_ERR_LAUNCH, "scan_lengths_static: hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices) return fail(CG_ERR_ARG, "scan_lengths_static: device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
+    if (!g_static_scratch[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p)
+            return fail(CG_ERR_LAUNCH, "scan_lengths_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+        g_static_scratch[dev] = p;
+    }
+    *ptr = g_static_scratch[dev];
+    return CG_OK;
+}
+
+}  // namespace
+
+// ======================================================================================
 // C ABI
 // ======================================================================================
 extern "C" {
 
 const char *cg_last_error(void) { return g_error; }
-int cg_abi_version(void) { return 3; }
+int cg_abi_version(void) { return 4; }
 
 int64_t cg_num_chunks(int64_t T, int64_t chunk_tokens)
 {
@@ -177,6 +216,20 @@ int cg_scan_lengths(const int32_t *lengths, int64_t n, int64_t *offsets, void *s
     if (n <= 0) return fail(CG_ERR_ARG, "scan: empty input");
     if (scratch_bytes < cg_scan_workspace(n)) return fail(CG_ERR_WORKSPACE, "scan: scratch too small");
     return launch_scan(lengths, n, INT_MAX, offsets, scratch, static_cast<hipStream_t>(stream));
+}
+
+int cg_scan_lengths_static(const int32_t *lengths, int64_t n, int64_t *offsets, void *stream)
+{
+    if (!lengths || !offsets) return fail(CG_ERR_ARG, "scan_lengths_static: null pointer");
+    if (n <= 0) return fail(CG_ERR_ARG, "scan_lengths_static: empty input");
+    if (n > kStaticScanMaxLengths)
+        return fail(CG_ERR_WORKSPACE, "scan_lengths_static: %lld lengths exceed the built-in scratch (at most %lld); "
+                                      "use cg_scan_lengths with a workspace", (long long)n, (long long)kStaticScanMaxLengths);
+    void *ptr = nullptr;
+    if (int rc = static_scratch(&ptr)) return rc;
+    // every partial sum the second and third kernel read is written by the first kernel of this
+    // same call, so nothing of the previous call's contents has to be cleared
+    return launch_scan(lengths, n, INT_MAX, offsets, ptr, static_cast<hipStream_t>(stream));
 }
 
 size_t cg_encode_kv_workspace(int64_t L, int64_t T, int64_t C, int64_t chunk_tokens)

@@ -156,6 +156,18 @@ size_t cg_scan_workspace(int64_t n);
 int cg_scan_lengths(const int32_t *lengths, int64_t n, int64_t *offsets,
                     void *scratch, size_t scratch_bytes, void *stream);
 
+/* cg_scan_lengths for callers that cannot allocate device memory and have no workspace to
+ * pass (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
+ * No counterpart in the reference.  Same results as cg_scan_lengths; the partial sums live
+ * in an array that is part of the library's device image (about 64 KiB on every GPU the
+ * library runs on, held until the process ends), so the call allocates and frees nothing.
+ * n <= CG_SCAN_STATIC_MAX_LENGTHS, CG_ERR_WORKSPACE otherwise.  All calls on one GPU share that
+ * array: two calls whose kernels overlap on the same GPU (different streams, or different
+ * threads on different streams) race; calls queued on one stream do not.  The first call on a
+ * device looks the array's address up (hipGetSymbolAddress) with that device current. */
+#define CG_SCAN_STATIC_MAX_LENGTHS (16 * 1024 * 1024)
+int cg_scan_lengths_static(const int32_t *lengths, int64_t n, int64_t *offsets, void *stream);
+
 /* decode_function_gpu + do_dequantize + the final cast and layout (decoder.py:
  * 77-112, 24-34, 159-173) for every chunk at once.
  * cdf, maxima, offsets, payload: as written by cg_encode_kv (maxima in max_dt);

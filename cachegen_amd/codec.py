@@ -263,14 +263,81 @@ def quantize_kv(kv, key_bins, value_bins, fmt="vllm"):
     return sym, maxima
 
 
-def encode_kv_levels(kv, levels, chunk_tokens=None, fmt="vllm", workspace=None):
-    """Encode the same KV cache at several quantization levels (the adaptive-streaming
-    use of the reference: src/utils.py:357-377 and run_adaptation.py:63-72 pre-encode every
-    chunk at QUANT_LEVEL 1..3).  `levels` is a list of (key_bins, value_bins); returns one
-    EncodedKV per level.  The workspace is shared, the results are independent."""
-    (L, T, H, D), _ = _kv_strides(kv, fmt)
+def encode_levels_workspace_bytes(num_layers, num_tokens, num_channels, chunk_tokens, num_levels):
+    return int(_lib.lib().cg_encode_kv_levels_workspace(num_layers, num_tokens, num_channels, chunk_tokens, num_levels))
+
+
+def encode_kv_levels(kv, levels, chunk_tokens=None, fmt="vllm", workspace=None, max_bins=None, out=None):
+    """Encode the same KV cache at several quantization levels from one read of the tensor (the
+    adaptive-streaming use of the reference: src/utils.py:357-377 and run_adaptation.py:63-72
+    pre-encode every chunk at QUANT_LEVEL 1..3, one serializer call per level).  `levels` is a
+    list of (key_bins, value_bins); `max_bins` an optional list of table sizes (default: each
+    level's largest bins value).  Returns one EncodedKV per level; they share the row maxima
+    (which do not depend on the level) and nothing else, and each equals what `encode_kv` gives
+    for that level.  `out`: a previous result of the same call, to reuse its tensors."""
+    import ctypes
+    if not kv.is_cuda:
+        raise RuntimeError("KV tensor should be on GPU")
+    if kv.dtype not in _DT:
+        raise RuntimeError("KV tensor must be float16 or bfloat16")
+    (L, T, H, D), (sl, skv, st, sh) = _kv_strides(kv, fmt)
+    C = H * D
     S = int(chunk_tokens) if chunk_tokens else T
-    ws_bytes = encode_workspace_bytes(L, T, H * D, S)
+    n = len(levels)
+    lib = _lib.lib()
+    if not 1 <= n <= 8:
+        raise RuntimeError("between 1 and 8 levels, got %d" % n)
+    dev = kv.device
+    bins = []
+    for kb, vb in levels:
+        if kb.numel() != L or vb.numel() != L:
+            raise RuntimeError("bins vectors must have one entry per layer (%d)" % L)
+        bins.append((kb.to(device=dev, dtype=torch.float32).contiguous(), vb.to(device=dev, dtype=torch.float32).contiguous()))
+    if max_bins is None:
+        max_bins = [int(max(float(kb.max()), float(vb.max()))) for kb, vb in levels]
+    if len(max_bins) != n:
+        raise RuntimeError("max_bins must have one entry per level")
+    nchunks = int(lib.cg_num_chunks(T, S))
+    nsub = int(lib.cg_num_subchunks(T, S))
+    nstreams = nsub * 2 * L * C
+    ws_bytes = int(lib.cg_encode_kv_levels_workspace(L, T, C, S, n))
     if workspace is None or workspace.numel() < ws_bytes:
-        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=kv.device)
-    return [encode_kv(kv, kb, vb, chunk_tokens=S, fmt=fmt, workspace=workspace) for kb, vb in levels]
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    if out is None:
+        maxima = torch.empty((2, L, T), dtype=kv.dtype, device=dev)
+        status = torch.empty(n, dtype=torch.int32, device=dev)
+        out = [EncodedKV(
+            cdf=torch.empty((nchunks, 2 * L, C, mb + 1), dtype=torch.int16, device=dev),
+            maxima=maxima,
+            lengths=torch.empty((nsub, 2 * L, C), dtype=torch.int32, device=dev),
+            offsets=torch.empty(nstreams + 1, dtype=torch.int64, device=dev),
+            payload=torch.empty(nstreams * MAX_TOKENS_PER_STREAM, dtype=torch.uint8, device=dev),
+            status=status[v:v + 1],
+            num_layers=L, num_tokens=T, num_heads=H, head_size=D, chunk_tokens=S, max_bins=mb)
+            for v, mb in enumerate(max_bins)]
+    else:
+        if len(out) != n:
+            raise RuntimeError("encode_kv_levels: `out` holds %d levels, this call %d" % (len(out), n))
+        for e, mb in zip(out, max_bins):
+            if (e.num_layers, e.num_tokens, e.num_heads, e.head_size, e.chunk_tokens, e.max_bins) != (L, T, H, D, S, mb) \
+                    or e.maxima.data_ptr() != out[0].maxima.data_ptr() or e.maxima.dtype != kv.dtype \
+                    or tuple(e.cdf.shape) != (nchunks, 2 * L, C, mb + 1) or e.lengths.numel() != nstreams:
+                raise RuntimeError("encode_kv_levels: `out` was made for another geometry")
+        if any(out[v].status.data_ptr() != out[0].status.data_ptr() + 4 * v for v in range(n)):
+            raise RuntimeError("encode_kv_levels: `out` must come from a previous encode_kv_levels call")
+
+    def ptrs(ctype, values):
+        return (ctype * n)(*values)
+
+    with torch.cuda.device(dev):
+        _lib.check(lib.cg_encode_kv_levels(
+            kv.data_ptr(), _DT[kv.dtype], L, T, H, D, sl, skv, st, sh, n,
+            ptrs(ctypes.c_void_p, [kb.data_ptr() for kb, _ in bins]), ptrs(ctypes.c_void_p, [vb.data_ptr() for _, vb in bins]),
+            ptrs(ctypes.c_int, max_bins), S,
+            ptrs(ctypes.c_void_p, [e.cdf.data_ptr() for e in out]), out[0].maxima.data_ptr(),
+            ptrs(ctypes.c_void_p, [e.lengths.data_ptr() for e in out]),
+            ptrs(ctypes.c_void_p, [e.offsets.data_ptr() for e in out]),
+            ptrs(ctypes.c_void_p, [e.payload.data_ptr() for e in out]),
+            ptrs(ctypes.c_int64, [e.payload.numel() for e in out]),
+            out[0].status.data_ptr(), workspace.data_ptr(), workspace.numel(), _stream()))
+    return out

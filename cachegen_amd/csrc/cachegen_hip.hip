@@ -82,7 +82,7 @@ int static_scratch(void **ptr)
 extern "C" {
 
 const char *cg_last_error(void) { return g_error; }
-int cg_abi_version(void) { return 4; }
+int cg_abi_version(void) { return 5; }
 
 int64_t cg_num_chunks(int64_t T, int64_t chunk_tokens)
 {
@@ -232,19 +232,158 @@ int cg_scan_lengths_static(const int32_t *lengths, int64_t n, int64_t *offsets, 
     return launch_scan(lengths, n, INT_MAX, offsets, ptr, static_cast<hipStream_t>(stream));
 }
 
+}  // extern "C"
+
+namespace {
+
+// Workspace of the fused encoder, carved in this order: `nlevels` symbol areas (a 256-token
+// slot per stream each), the coder's scratch tiles, and the small arrays of the two running sums.
+struct EncodeWorkspace {
+    size_t symbols_bytes;       // one level's symbols
+    uint8_t *symbols, *scratch;
+    void *scan_scratch, *tile_scan_scratch;
+    int32_t *tile_sums;
+    int64_t *tile_base;
+    int64_t nsub, nstreams, ntiles;
+    size_t total;
+
+    EncodeWorkspace(void *base, int64_t L, int64_t T, int64_t C, int64_t chunk_tokens, int nlevels)
+    {
+        nsub = cg_num_subchunks(T, chunk_tokens);
+        nstreams = nsub * 2 * L * C;
+        ntiles = ceil_div(nstreams, kSlotTile);
+        symbols_bytes = align_up((size_t)nstreams * kSub, 256);
+        uint8_t *ws = static_cast<uint8_t *>(base);
+        symbols = ws;
+        ws += symbols_bytes * (size_t)nlevels;
+        scratch = ws;           // kStreamCap bytes per stream, in tiles of kSlotTile word-interleaved streams
+        ws += (size_t)ntiles * kSlotTile * kStreamCap;
+        scan_scratch = ws;
+        ws += cg_scan_workspace(nstreams);
+        tile_sums = reinterpret_cast<int32_t *>(ws);           // bytes per tile of streams
+        ws += align_up((size_t)ntiles * sizeof(int32_t), 256);
+        tile_base = reinterpret_cast<int64_t *>(ws);           // their running sums
+        ws += align_up((size_t)(ntiles + 1) * sizeof(int64_t), 256);
+        tile_scan_scratch = ws;
+        ws += cg_scan_workspace(ntiles);
+        total = (size_t)(ws - static_cast<uint8_t *>(base));
+    }
+};
+
+}  // namespace
+
+extern "C" {
+
 size_t cg_encode_kv_workspace(int64_t L, int64_t T, int64_t C, int64_t chunk_tokens)
 {
-    const int64_t nsub = cg_num_subchunks(T, chunk_tokens);
-    const int64_t nstreams = nsub * 2 * L * C;
-    size_t total = align_up((size_t)nstreams * kSub, 256);        // symbols: a 256-token slot per stream
-    total += (size_t)ceil_div(nstreams, kSlotTile) * kSlotTile * kStreamCap;   // encoder scratch: whole tiles of slots
-    total += cg_scan_workspace(nstreams);
-    const int64_t ntiles = ceil_div(nstreams, kSlotTile);
-    total += align_up((size_t)ntiles * sizeof(int32_t), 256);          // bytes per tile of streams
-    total += align_up((size_t)(ntiles + 1) * sizeof(int64_t), 256);    // their running sums
-    total += cg_scan_workspace(ntiles);
-    return total;
+    return EncodeWorkspace(nullptr, L, T, C, chunk_tokens, 1).total;
 }
+
+size_t cg_encode_kv_levels_workspace(int64_t L, int64_t T, int64_t C, int64_t chunk_tokens, int nlevels)
+{
+    if (nlevels < 1 || nlevels > CG_MAX_LEVELS) return 0;
+    return EncodeWorkspace(nullptr, L, T, C, chunk_tokens, nlevels).total;
+}
+
+}  // extern "C"
+
+namespace {
+
+// What one quantization level's outputs are.
+struct LevelOut {
+    const float *key_bins, *value_bins;
+    int max_bins;
+    int16_t *cdf;
+    int32_t *lengths;
+    int64_t *offsets;
+    uint8_t *payload;
+    int64_t payload_cap;
+    int32_t *status;
+};
+
+// Tables, streams and payload of one level from its symbols (packed words `sym4`, or byte
+// symbols [2L, T, C]): calculate_cdf + encode_fast_new + collect_bytes for every chunk
+// (encoder.py:265-292, 209-222).
+int code_and_compact(const LevelOut &o, const uint32_t *sym4, const uint8_t *sym_bytes, const EncodeWorkspace &w,
+                     int64_t L, int64_t T, int64_t C, int64_t chunk_tokens, hipStream_t s)
+{
+    const int64_t rows = 2 * L;
+    const int lp = o.max_bins + 1;
+    uint16_t *tables = reinterpret_cast<uint16_t *>(o.cdf);
+    clear_status_kernel<<<1, 1, 0, s>>>(o.status);
+
+    const int block = pick_block(C, lp);
+    EncodeArgs a;
+    memset(&a, 0, sizeof(a));
+    a.cdf = tables;
+    a.lp = lp;
+    a.nsub = w.nsub;
+    a.out = w.scratch;
+    a.cap = kStreamCap;
+    a.lengths = o.lengths;
+    a.status = o.status;
+    a.key_bins = o.key_bins;
+    a.value_bins = o.value_bins;
+    a.L = L;
+    int64_t nblocks;
+    if (int rc = make_grid(rows, C, T, chunk_tokens, w.nsub, block, a.sg, nblocks)) return rc;
+    const size_t shmem = (size_t)lp * (block + 2) * sizeof(uint16_t);      // TableStride<BS>::k16 per entry
+    const dim3 grid((unsigned)nblocks), blk(block);
+    // when every encoder block is exactly one tile of the scratch, the blocks leave their byte
+    // counts behind and the compaction computes the stream offsets itself
+    const bool fused_scan = block == kSlotTile && C % kSlotTile == 0;
+    a.tile_sums = fused_scan ? w.tile_sums : nullptr;
+
+    if (sym4) {
+        // four tokens per word, read by one lane per channel
+        a.sym4 = sym4;
+        if (chunk_tokens <= kSub) {
+            // one sub-chunk per chunk: the encoder builds the tables itself
+            if (fused_scan) encode_streams_kernel<kSlotTile, true, true, true, true, true><<<grid, blk, shmem, s>>>(a);
+            else CG_DISPATCH_BS(block, (encode_streams_kernel<BS, true, true, true, true><<<grid, blk, shmem, s>>>(a)));
+        } else {
+            if (int rc = launch_cdf(nullptr, sym4, w.nsub, rows, T, C, 0, 0, 0, o.max_bins, chunk_tokens, tables, s)) return rc;
+            if (fused_scan) encode_streams_kernel<kSlotTile, true, true, false, true, true><<<grid, blk, shmem, s>>>(a);
+            else CG_DISPATCH_BS(block, (encode_streams_kernel<BS, true, true, false, true><<<grid, blk, shmem, s>>>(a)));
+        }
+    } else {
+        // any shape or alignment: byte symbols [2L, T, C]
+        if (int rc = launch_cdf(sym_bytes, nullptr, 0, rows, T, C, T * C, C, 1, o.max_bins, chunk_tokens, tables, s)) return rc;
+        a.sym = sym_bytes;
+        a.s0 = T * C;
+        a.s1 = C;
+        a.s2 = 1;
+        CG_DISPATCH_BS(block, (encode_streams_kernel<BS, true, false, false, true><<<grid, blk, shmem, s>>>(a)));
+    }
+    if (int rc = check_launch("encode_kv")) return rc;
+
+    const int64_t cblocks = ceil_div(w.nstreams, kCompactStreams);
+    if (cblocks > INT_MAX) return fail(CG_ERR_ARG, "encode_kv: too many streams");
+    const int32_t skew = (int32_t)(reinterpret_cast<uintptr_t>(o.payload) & 3u);
+    if (fused_scan) {
+        if (int rc = launch_scan(w.tile_sums, cblocks, INT_MAX, w.tile_base, w.tile_scan_scratch, s)) return rc;
+        compact_streams_kernel<true><<<dim3((unsigned)cblocks), dim3(256), 0, s>>>(
+            w.scratch, kStreamCap, o.offsets, o.lengths, w.tile_base, w.nstreams, o.payload, o.payload_cap, skew, o.status);
+    } else {
+        if (int rc = launch_scan(o.lengths, w.nstreams, kStreamCap, o.offsets, w.scan_scratch, s)) return rc;
+        compact_streams_kernel<false><<<dim3((unsigned)cblocks), dim3(256), 0, s>>>(
+            w.scratch, kStreamCap, o.offsets, nullptr, nullptr, w.nstreams, o.payload, o.payload_cap, skew, o.status);
+    }
+    return check_launch("compact");
+}
+
+int check_kv_geometry(const char *what, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D, int64_t chunk_tokens)
+{
+    if (int rc = check_dt(kv_dt, what)) return rc;
+    if (L <= 0 || T <= 0 || H <= 0 || D <= 0) return fail(CG_ERR_ARG, "%s: empty input", what);
+    if (chunk_tokens <= 0) return fail(CG_ERR_ARG, "%s: chunk_tokens must be positive", what);
+    if (chunk_tokens > 65535) return fail(CG_ERR_ARG, "%s: at most 65535 tokens per chunk (16-bit counters)", what);
+    return CG_OK;
+}
+
+}  // namespace
+
+extern "C" {
 
 int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D, int64_t sl,
                  int64_t skv, int64_t st, int64_t sh, const float *key_bins, const float *value_bins,
@@ -254,102 +393,75 @@ int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int
 {
     if (!kv || !key_bins || !value_bins || !cdf || !maxima || !lengths || !offsets || !payload || !status || !workspace)
         return fail(CG_ERR_ARG, "encode_kv: null pointer");
-    if (int rc = check_dt(kv_dt, "encode_kv")) return rc;
-    if (L <= 0 || T <= 0 || H <= 0 || D <= 0) return fail(CG_ERR_ARG, "encode_kv: empty input");
-    if (chunk_tokens <= 0) return fail(CG_ERR_ARG, "encode_kv: chunk_tokens must be positive");
-    if (chunk_tokens > 65535) return fail(CG_ERR_ARG, "encode_kv: at most 65535 tokens per chunk (16-bit counters)");
+    if (int rc = check_kv_geometry("encode_kv", kv_dt, L, T, H, D, chunk_tokens)) return rc;
     if (int rc = check_lp(max_bins + 1, "encode_kv")) return rc;
     if (delta_group < 0 || delta_group > kSub) return fail(CG_ERR_ARG, "encode_kv: delta_group must be in [0, %d]", kSub);
-    const int64_t C = H * D, rows = 2 * L;
-    const int64_t nsub = cg_num_subchunks(T, chunk_tokens);
-    const int64_t nstreams = nsub * rows * C;
-    if (workspace_bytes < cg_encode_kv_workspace(L, T, C, chunk_tokens)) return fail(CG_ERR_WORKSPACE, "encode_kv: workspace too small");
+    const int64_t C = H * D;
+    const EncodeWorkspace w(workspace, L, T, C, chunk_tokens, 1);
+    if (workspace_bytes < w.total) return fail(CG_ERR_WORKSPACE, "encode_kv: workspace too small");
     if (!aligned_to(workspace, 256)) return fail(CG_ERR_ARG, "encode_kv: workspace must be 256-byte aligned");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const int lp = max_bins + 1;
-
-    uint8_t *ws = static_cast<uint8_t *>(workspace);
-    uint8_t *symbols = ws;
-    ws += align_up((size_t)nstreams * kSub, 256);
-    uint8_t *scratch = ws;     // kStreamCap bytes per stream, in tiles of kSlotTile word-interleaved streams
-    ws += (size_t)ceil_div(nstreams, kSlotTile) * kSlotTile * kStreamCap;
-    void *scan_scratch = ws;
-    ws += cg_scan_workspace(nstreams);
-    const int64_t ntiles = ceil_div(nstreams, kSlotTile);
-    int32_t *tile_sums = reinterpret_cast<int32_t *>(ws);
-    ws += align_up((size_t)ntiles * sizeof(int32_t), 256);
-    int64_t *tile_base = reinterpret_cast<int64_t *>(ws);
-    ws += align_up((size_t)(ntiles + 1) * sizeof(int64_t), 256);
-    void *tile_scan_scratch = ws;
-    uint16_t *tables = reinterpret_cast<uint16_t *>(cdf);
-
-    clear_status_kernel<<<1, 1, 0, s>>>(status);
-
-    const int block = pick_block(C, lp);
-    EncodeArgs a;
-    memset(&a, 0, sizeof(a));
-    a.cdf = tables;
-    a.lp = lp;
-    a.nsub = nsub;
-    a.out = scratch;
-    a.cap = kStreamCap;
-    a.lengths = lengths;
-    a.status = status;
-    a.key_bins = key_bins;
-    a.value_bins = value_bins;
-    a.L = L;
-    int64_t nblocks;
-    if (int rc = make_grid(rows, C, T, chunk_tokens, nsub, block, a.sg, nblocks)) return rc;
-    const size_t shmem = (size_t)lp * (block + 2) * sizeof(uint16_t);      // TableStride<BS>::k16 per entry
-    const dim3 grid((unsigned)nblocks), blk(block);
-    // when every encoder block is exactly one tile of the scratch, the blocks leave their byte
-    // counts behind and the compaction computes the stream offsets itself
-    const bool fused_scan = block == kSlotTile && C % kSlotTile == 0;
-    a.tile_sums = fused_scan ? tile_sums : nullptr;
+    const LevelOut o = {key_bins, value_bins, max_bins, cdf, lengths, offsets, payload, payload_cap, status};
 
     const bool packed = kv_vectorizable(kv, D, C, sl, skv, st, sh) && C % 8 == 0;
     if (delta_group > 0 && !packed)
         return fail(CG_ERR_ARG, "encode_kv: delta groups need head sizes and strides that are multiples of 8 and a 16-byte aligned tensor");
     if (packed) {
-        // four tokens per word, read by one lane per channel
-        uint32_t *sym4 = reinterpret_cast<uint32_t *>(symbols);
+        uint32_t *sym4 = reinterpret_cast<uint32_t *>(w.symbols);
         if (int rc = launch_quantize_pack(kv, kv_dt, L, T, H, D, sl, skv, st, sh, key_bins, value_bins, sym4,
-                                          maxima, nsub, chunk_tokens, delta_group, s)) return rc;
-        a.sym4 = sym4;
-        if (chunk_tokens <= kSub) {
-            // one sub-chunk per chunk: the encoder builds the tables itself
-            if (fused_scan) encode_streams_kernel<kSlotTile, true, true, true, true, true><<<grid, blk, shmem, s>>>(a);
-            else CG_DISPATCH_BS(block, (encode_streams_kernel<BS, true, true, true, true><<<grid, blk, shmem, s>>>(a)));
-        } else {
-            if (int rc = launch_cdf(nullptr, sym4, nsub, rows, T, C, 0, 0, 0, max_bins, chunk_tokens, tables, s)) return rc;
-            if (fused_scan) encode_streams_kernel<kSlotTile, true, true, false, true, true><<<grid, blk, shmem, s>>>(a);
-            else CG_DISPATCH_BS(block, (encode_streams_kernel<BS, true, true, false, true><<<grid, blk, shmem, s>>>(a)));
-        }
-    } else {
-        // any shape or alignment: byte symbols [2L, T, C]
-        if (int rc = launch_quantize(kv, kv_dt, L, T, H, D, sl, skv, st, sh, key_bins, value_bins, symbols, maxima, s)) return rc;
-        if (int rc = launch_cdf(symbols, nullptr, 0, rows, T, C, T * C, C, 1, max_bins, chunk_tokens, tables, s)) return rc;
-        a.sym = symbols;
-        a.s0 = T * C;
-        a.s1 = C;
-        a.s2 = 1;
-        CG_DISPATCH_BS(block, (encode_streams_kernel<BS, true, false, false, true><<<grid, blk, shmem, s>>>(a)));
+                                          maxima, w.nsub, chunk_tokens, delta_group, s)) return rc;
+        return code_and_compact(o, sym4, nullptr, w, L, T, C, chunk_tokens, s);
     }
-    if (int rc = check_launch("encode_kv")) return rc;
+    if (int rc = launch_quantize(kv, kv_dt, L, T, H, D, sl, skv, st, sh, key_bins, value_bins, w.symbols, maxima, s)) return rc;
+    return code_and_compact(o, nullptr, w.symbols, w, L, T, C, chunk_tokens, s);
+}
 
-    const int64_t cblocks = ceil_div(nstreams, kCompactStreams);
-    if (cblocks > INT_MAX) return fail(CG_ERR_ARG, "encode_kv: too many streams");
-    const int32_t skew = (int32_t)(reinterpret_cast<uintptr_t>(payload) & 3u);
-    if (fused_scan) {
-        if (int rc = launch_scan(tile_sums, cblocks, INT_MAX, tile_base, tile_scan_scratch, s)) return rc;
-        compact_streams_kernel<true><<<dim3((unsigned)cblocks), dim3(256), 0, s>>>(
-            scratch, kStreamCap, offsets, lengths, tile_base, nstreams, payload, payload_cap, skew, status);
-    } else {
-        if (int rc = launch_scan(lengths, nstreams, kStreamCap, offsets, scan_scratch, s)) return rc;
-        compact_streams_kernel<false><<<dim3((unsigned)cblocks), dim3(256), 0, s>>>(
-            scratch, kStreamCap, offsets, nullptr, nullptr, nstreams, payload, payload_cap, skew, status);
+int cg_encode_kv_levels(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D, int64_t sl,
+                        int64_t skv, int64_t st, int64_t sh, int nlevels, const float *const *key_bins,
+                        const float *const *value_bins, const int *max_bins, int64_t chunk_tokens,
+                        int16_t *const *cdf, void *maxima, int32_t *const *lengths, int64_t *const *offsets,
+                        uint8_t *const *payload, const int64_t *payload_cap, int32_t *status,
+                        void *workspace, size_t workspace_bytes, void *stream)
+{
+    if (!kv || !key_bins || !value_bins || !max_bins || !cdf || !maxima || !lengths || !offsets || !payload ||
+        !payload_cap || !status || !workspace)
+        return fail(CG_ERR_ARG, "encode_kv_levels: null pointer");
+    if (nlevels < 1 || nlevels > CG_MAX_LEVELS)
+        return fail(CG_ERR_ARG, "encode_kv_levels: between 1 and %d levels, got %d", CG_MAX_LEVELS, nlevels);
+    if (int rc = check_kv_geometry("encode_kv_levels", kv_dt, L, T, H, D, chunk_tokens)) return rc;
+    for (int v = 0; v < nlevels; ++v) {
+        if (!key_bins[v] || !value_bins[v] || !cdf[v] || !lengths[v] || !offsets[v] || !payload[v])
+            return fail(CG_ERR_ARG, "encode_kv_levels: null pointer for level %d", v);
+        if (int rc = check_lp(max_bins[v] + 1, "encode_kv_levels")) return rc;
     }
-    return check_launch("compact");
+    const int64_t C = H * D;
+    const EncodeWorkspace w(workspace, L, T, C, chunk_tokens, nlevels);
+    if (workspace_bytes < w.total) return fail(CG_ERR_WORKSPACE, "encode_kv_levels: workspace too small");
+    if (!aligned_to(workspace, 256)) return fail(CG_ERR_ARG, "encode_kv_levels: workspace must be 256-byte aligned");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+
+    const bool packed = kv_vectorizable(kv, D, C, sl, skv, st, sh) && C % 8 == 0;
+    if (packed) {
+        // one pass over the tensor: every row is loaded once, its maximum found once, and its
+        // symbols written once per level
+        uint32_t *sym4 = reinterpret_cast<uint32_t *>(w.symbols);
+        if (int rc = launch_quantize_pack(kv, kv_dt, L, T, H, D, sl, skv, st, sh, nullptr, nullptr, sym4, maxima,
+                                          w.nsub, chunk_tokens, 0, s, nlevels, key_bins, value_bins,
+                                          (int64_t)(w.symbols_bytes / 4))) return rc;
+    }
+    for (int v = 0; v < nlevels; ++v) {
+        const LevelOut o = {key_bins[v], value_bins[v], max_bins[v], cdf[v], lengths[v], offsets[v],
+                            payload[v], payload_cap[v], status + v};
+        uint8_t *symbols = w.symbols + (size_t)v * w.symbols_bytes;
+        if (packed) {
+            if (int rc = code_and_compact(o, reinterpret_cast<uint32_t *>(symbols), nullptr, w, L, T, C, chunk_tokens, s)) return rc;
+        } else {
+            // shapes the vector loads cannot take: one plain quantization pass per level
+            if (int rc = launch_quantize(kv, kv_dt, L, T, H, D, sl, skv, st, sh, key_bins[v], value_bins[v], symbols, maxima, s)) return rc;
+            if (int rc = code_and_compact(o, nullptr, symbols, w, L, T, C, chunk_tokens, s)) return rc;
+        }
+    }
+    return CG_OK;
 }
 
 int cg_decode_kv(const int16_t *cdf, int max_bins, const void *maxima, int max_dt, const int64_t *offsets,

@@ -151,17 +151,35 @@ void launch_quantize_pack_nu(const PackedQuantArgs &a, int64_t nblocks, hipStrea
         else quantize_pack_delta_kernel<DT, HC, 8><<<grid, block, 0, stream>>>(a);
         return;
     }
+    if (a.nlevels > 0) {
+        if (a.nunits <= 128) quantize_pack_kernel<DT, HC, 2, true><<<grid, block, 0, stream>>>(a);
+        else if (a.nunits <= 256) quantize_pack_kernel<DT, HC, 4, true><<<grid, block, 0, stream>>>(a);
+        else quantize_pack_kernel<DT, HC, 8, true><<<grid, block, 0, stream>>>(a);
+        return;
+    }
     if (a.nunits <= 128) quantize_pack_kernel<DT, HC, 2><<<grid, block, 0, stream>>>(a);
     else if (a.nunits <= 256) quantize_pack_kernel<DT, HC, 4><<<grid, block, 0, stream>>>(a);
     else quantize_pack_kernel<DT, HC, 8><<<grid, block, 0, stream>>>(a);
 }
 
+// nlevels > 0: key_bins_lv / value_bins_lv hold that many bins vectors and level v's words go
+// to sym4 + v * level_words (one read of the tensor for all levels); nlevels == 0: one level,
+// key_bins / value_bins.
 int launch_quantize_pack(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D,
                          int64_t sl, int64_t skv, int64_t st, int64_t sh, const float *key_bins,
                          const float *value_bins, uint32_t *sym4, void *maxima, int64_t nsub,
-                         int64_t S, int delta_group, hipStream_t stream)
+                         int64_t S, int delta_group, hipStream_t stream, int nlevels = 0,
+                         const float *const *key_bins_lv = nullptr, const float *const *value_bins_lv = nullptr,
+                         int64_t level_words = 0)
 {
     PackedQuantArgs a;
+    memset(&a, 0, sizeof(a));
+    a.nlevels = nlevels;
+    for (int v = 0; v < nlevels; ++v) {
+        a.key_bins_lv[v] = key_bins_lv[v];
+        a.value_bins_lv[v] = value_bins_lv[v];
+    }
+    a.level_words = level_words;
     a.kv = static_cast<const uint16_t *>(kv);
     a.L = L;
     a.sl = sl;

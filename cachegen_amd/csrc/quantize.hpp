@@ -151,11 +151,18 @@ __global__ __launch_bounds__(256) void quantize_kv_generic_kernel(
 // ------------------------------------------------------------------------------------
 constexpr int kWordsPerSub = kSub / 4;
 
+constexpr int kMaxLevels = CG_MAX_LEVELS;
+
 struct PackedQuantArgs {
     const uint16_t *kv;
     int64_t L, sl, skv, st, sh;
     int32_t D;
     const float *key_bins, *value_bins;
+    // several quantization levels from one read of the tensor (MULTI kernels): level v uses
+    // key_bins_lv[v] / value_bins_lv[v] and writes its words level_words * v further on
+    int32_t nlevels;
+    const float *key_bins_lv[kMaxLevels], *value_bins_lv[kMaxLevels];
+    int64_t level_words;
     uint32_t *sym4;
     uint16_t *maxima;       // [2L, T]
     int32_t nunits;         // C / 8
@@ -167,7 +174,10 @@ struct PackedQuantArgs {
 // One wavefront quantizes four consecutive tokens of one row (encoder.py:42-59) and
 // writes, per channel, one word holding the four symbols: 32 contiguous bytes per lane
 // and unit, 2 KB per wave and store pair.
-template <int DT, bool HEADS_CONTIGUOUS, int NU>
+// MULTI: the rows are loaded and their maxima found once, then quantized at each of
+// a.nlevels levels (the adaptive-streaming use: run_adaptation.py:63-72 encodes every chunk
+// at QUANT_LEVEL 1..3); the maxima do not depend on the level.
+template <int DT, bool HEADS_CONTIGUOUS, int NU, bool MULTI = false>
 __global__ __launch_bounds__(256) void quantize_pack_kernel(PackedQuantArgs a)
 {
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -183,12 +193,10 @@ __global__ __launch_bounds__(256) void quantize_pack_kernel(PackedQuantArgs a)
     if (tt0 >= n) return;
     const int nvalid = (n - tt0) < 4 ? (n - tt0) : 4;
     const int64_t kvi = row / a.L, l = row - kvi * a.L;
-    const float bins = (kvi ? a.value_bins : a.key_bins)[l];
-    const float maxq = floorf(bins * 0.5f) - 1.0f;
     const uint16_t *base = a.kv + l * a.sl + kvi * a.skv + (t0 + tt0) * a.st;
 
     uint4 regs[4][NU];
-    float factor[4];
+    float rowmax[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         uint32_t m = 0;
@@ -211,35 +219,43 @@ __global__ __launch_bounds__(256) void quantize_pack_kernel(PackedQuantArgs a)
         m = (m & 0xFFFFu) > (m >> 16) ? (m & 0xFFFFu) : (m >> 16);
         m = wave_max_u32(m);
         if (j < nvalid && lane == 0) a.maxima[row * a.g.T + t0 + tt0 + j] = (uint16_t)m;
-        // rows past the end of the sub-chunk are all zero: 0 * inf = NaN -> symbol byte 0
-        factor[j] = __fdiv_rn(maxq, load16f<DT>(m));
+        rowmax[j] = load16f<DT>(m);
     }
 
     const int64_t C = (int64_t)a.nunits * 8;
     uint32_t *out = a.sym4 + ((row * a.nsub + sub) * kWordsPerSub + tq) * C;
+    const int nlevels = MULTI ? a.nlevels : 1;
+    for (int lv = 0; lv < nlevels; ++lv, out += a.level_words) {
+        const float bins = MULTI ? (kvi ? a.value_bins_lv[lv] : a.key_bins_lv[lv])[l] : (kvi ? a.value_bins : a.key_bins)[l];
+        const float maxq = floorf(bins * 0.5f) - 1.0f;
+        float factor[4];
+        // rows past the end of the sub-chunk are all zero: 0 * inf = NaN -> symbol byte 0
 #pragma unroll
-    for (int i = 0; i < NU; ++i) {
-        const int u = lane + 64 * i;
-        if (u < a.nunits) {
-            uint32_t words[8];
+        for (int j = 0; j < 4; ++j) factor[j] = __fdiv_rn(maxq, rowmax[j]);
 #pragma unroll
-            for (int k = 0; k < 8; ++k) {
-                uint32_t w = 0;
+        for (int i = 0; i < NU; ++i) {
+            const int u = lane + 64 * i;
+            if (u < a.nunits) {
+                uint32_t words[8];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const uint32_t src = k < 2 ? regs[j][i].x : k < 4 ? regs[j][i].y
-                                       : k < 6 ? regs[j][i].z : regs[j][i].w;
-                    const uint32_t bits = (k & 1) ? (src >> 16) : (src & 0xFFFFu);
-                    const float v = load16f<DT>(bits);
-                    const float s = __fadd_rn(__fmul_rn(v, factor[j]), maxq);
-                    const float r = fmaxf(__builtin_rintf(s), 0.0f);     // NaN -> 0
-                    w = __builtin_amdgcn_cvt_pk_u8_f32(r, (uint32_t)j, w);
+                for (int k = 0; k < 8; ++k) {
+                    uint32_t w = 0;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const uint32_t src = k < 2 ? regs[j][i].x : k < 4 ? regs[j][i].y
+                                           : k < 6 ? regs[j][i].z : regs[j][i].w;
+                        const uint32_t bits = (k & 1) ? (src >> 16) : (src & 0xFFFFu);
+                        const float v = load16f<DT>(bits);
+                        const float s = __fadd_rn(__fmul_rn(v, factor[j]), maxq);
+                        const float r = fmaxf(__builtin_rintf(s), 0.0f);     // NaN -> 0
+                        w = __builtin_amdgcn_cvt_pk_u8_f32(r, (uint32_t)j, w);
+                    }
+                    words[k] = w;
                 }
-                words[k] = w;
+                uint4 *dst = reinterpret_cast<uint4 *>(out + (int64_t)u * 8);
+                dst[0] = make_uint4(words[0], words[1], words[2], words[3]);
+                dst[1] = make_uint4(words[4], words[5], words[6], words[7]);
             }
-            uint4 *dst = reinterpret_cast<uint4 *>(out + (int64_t)u * 8);
-            dst[0] = make_uint4(words[0], words[1], words[2], words[3]);
-            dst[1] = make_uint4(words[4], words[5], words[6], words[7]);
         }
     }
 }

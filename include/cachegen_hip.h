@@ -35,6 +35,7 @@ extern "C" {
 
 #define CG_MAX_TOKENS_PER_STREAM 256 /* cachegen_basics.py:8, enc_new.cu:9-15 */
 #define CG_MAX_LP 129                /* table length limit of this library (reference: 48 / 64) */
+#define CG_MAX_LEVELS 8              /* quantization levels one cg_encode_kv_levels call takes */
 
 /* Message for the last error returned on this thread ("" if none). */
 const char *cg_last_error(void);
@@ -148,6 +149,32 @@ int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int
                  int16_t *cdf, void *maxima, int32_t *lengths, int64_t *offsets,
                  uint8_t *payload, int64_t payload_cap, int32_t *status,
                  void *workspace, size_t workspace_bytes, void *stream);
+
+/* The same KV cache encoded at `nlevels` quantization levels from ONE read of the tensor: the
+ * adaptive-streaming use of the reference, which pre-encodes every chunk at QUANT_LEVEL 1..3
+ * by calling the serializer once per level (run_adaptation.py:63-72, src/utils.py:357-377).
+ * Every row is loaded once and its maximum found once; its symbols are written once per level
+ * and each level is then coded exactly as cg_encode_kv codes it, so level v's tables, lengths,
+ * offsets and payload are byte-identical to a cg_encode_kv call with key_bins[v],
+ * value_bins[v], max_bins[v].
+ * key_bins, value_bins   HOST arrays of nlevels device pointers (float32 [L] each)
+ * max_bins               HOST array of nlevels ints
+ * cdf, lengths, offsets, payload   HOST arrays of nlevels device pointers, shaped as in
+ *                        cg_encode_kv (cdf[v]: [nchunks, 2L, C, max_bins[v]+1]); payload_cap
+ *                        a HOST array of nlevels capacities
+ * maxima                 device 16-bit [2, L, T]: the row maxima do not depend on the level
+ * status                 device int32 [nlevels]
+ * workspace              cg_encode_kv_levels_workspace(...) bytes, 256-aligned
+ * 1 <= nlevels <= CG_MAX_LEVELS.  Tensors whose head size or strides are not multiples of 8
+ * are quantized once per level instead. */
+size_t cg_encode_kv_levels_workspace(int64_t L, int64_t T, int64_t C, int64_t chunk_tokens, int nlevels);
+int cg_encode_kv_levels(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D,
+                        int64_t sl, int64_t skv, int64_t st, int64_t sh,
+                        int nlevels, const float *const *key_bins, const float *const *value_bins,
+                        const int *max_bins, int64_t chunk_tokens,
+                        int16_t *const *cdf, void *maxima, int32_t *const *lengths,
+                        int64_t *const *offsets, uint8_t *const *payload, const int64_t *payload_cap,
+                        int32_t *status, void *workspace, size_t workspace_bytes, void *stream);
 
 /* Exclusive running sum of stream lengths: offsets[0] = 0, offsets[i+1] =
  * offsets[i] + lengths[i] (the inclusive sums of decoder.py:70 are offsets[1:]).

@@ -18,7 +18,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), name
     assert declared == set(_lib.SIGNATURES), declared ^ set(_lib.SIGNATURES)
-    assert lib.cg_abi_version() == 4
+    assert lib.cg_abi_version() == 5
     assert lib.cg_last_error() == b""
 
 

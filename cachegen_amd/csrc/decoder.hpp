@@ -34,6 +34,8 @@ namespace {
 
 // The most bits one symbol can move for a table without zero-width entries.
 constexpr uint32_t kSymbolBits = 18;
+// Symbols between two unconditional top-ups of the bit window.
+constexpr int kSymbolsPerTopUp = 8;
 
 struct BitReader {
     // Words are fetched with buffer loads: the descriptor (uniform over the wavefront) covers
@@ -325,15 +327,16 @@ __device__ __forceinline__ void decode_lane(const DecodeArgs &a, DecodeLane &s, 
         s.bound_lo = 0;
         s.bound_hi = 0;
     }
-    for (int i0 = 0; i0 < n; i0 += 4, rmp += 4) {
-        // the maxima of the next four token rows (the array is padded to a multiple of four)
-        float rm[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-        if (OUT != OUT_SYMBOLS) {
+    // the window is topped up at the head of every group of kGroup symbols and, inside a
+    // group, only when a symbol has left it short of bits
+    constexpr int kGroup = kSymbolsPerTopUp;
+    for (int i0 = 0; i0 < n; i0 += kGroup, rmp += kGroup) {
+        // the maxima of the group's token rows (the array is padded to a whole group)
+        float rm[kGroup];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) rm[j] = rmp[j];
-        }
+        for (int j = 0; j < kGroup; ++j) rm[j] = OUT != OUT_SYMBOLS ? rmp[j] : 0.0f;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < kGroup; ++j) {
             const int i = i0 + j;
             if (i >= n) break;
             if (j == 0) s.rd.top_up();
@@ -355,26 +358,37 @@ __global__ __launch_bounds__(BS) void decode_streams_kernel(DecodeArgs a)
     const int lp = LOG2 >= 0 ? (1 << LOG2) + 1 : a.lp;
     char *rows = reinterpret_cast<char *>(smem);
     float *rowmax = reinterpret_cast<float *>(rows + lp * kRow);     // one per token of the sub-chunk
-    const int64_t ch0 = id.ch - tid;
     {
-        // entry 0 of a table is 0 by construction (cal_cdf.cu:29-49 counts into hist[sym+1]);
-        // it is stored as 0 whatever the input holds so that the walk back always ends
-        const uint16_t *src = a.cdf + ((id.chunk * a.sg.rows + id.row) * a.sg.nc + ch0) * lp;
-        const int64_t nvalid = (a.sg.nc - ch0 < BS) ? (a.sg.nc - ch0) : BS;
-        const int total = (int)nvalid * lp;
-        TableWalk w(tid, BS, lp);
-        // sixteen loads are issued before the first value is needed: one trip to memory per
-        // sixteen table entries of a lane instead of one per entry
-        constexpr int kBatch = 16;
-        for (int i0 = tid; i0 < total; i0 += kBatch * BS) {
-            uint16_t v[kBatch];
+        // Every lane copies its own table (lp consecutive 16-bit entries) into its LDS column:
+        // loads and LDS writes with immediate offsets, no address arithmetic per entry; the
+        // lanes of a wavefront read neighbouring tables, so each cache line is fetched once.
+        // Entry 0 of a table is 0 by construction (cal_cdf.cu:29-49 counts into hist[sym+1]);
+        // it is stored as 0 whatever the input holds so that the walk back always ends.
+        const uint16_t *mine = a.cdf + ((id.chunk * a.sg.rows + id.row) * a.sg.nc + id.ch) * lp;
+        char *column = rows + 2 * tid;
+        if (id.active) {
+            *reinterpret_cast<uint16_t *>(column) = 0;
+            constexpr int kBatch = 16;      // loads in flight per lane
+            if (LOG2 >= 0) {
 #pragma unroll
-            for (int j = 0; j < kBatch; ++j) v[j] = i0 + j * BS < total ? src[i0 + j * BS] : (uint16_t)0;
+                for (int e0 = 1; e0 < lp; e0 += kBatch) {
+                    uint16_t v[kBatch];
 #pragma unroll
-            for (int j = 0; j < kBatch; ++j) {
-                if (i0 + j * BS < total)
-                    *reinterpret_cast<uint16_t *>(rows + w.e * kRow + 2 * w.c) = w.e == 0 ? (uint16_t)0 : v[j];
-                w.next(lp);
+                    for (int j = 0; j < kBatch; ++j)
+                        if (e0 + j < lp) v[j] = mine[e0 + j];
+#pragma unroll
+                    for (int j = 0; j < kBatch; ++j)
+                        if (e0 + j < lp) *reinterpret_cast<uint16_t *>(column + (e0 + j) * kRow) = v[j];
+                }
+            } else {
+                for (int e0 = 1; e0 < lp; e0 += kBatch) {
+                    uint16_t v[kBatch];
+#pragma unroll
+                    for (int j = 0; j < kBatch; ++j) v[j] = e0 + j < lp ? mine[e0 + j] : (uint16_t)0;
+#pragma unroll
+                    for (int j = 0; j < kBatch; ++j)
+                        if (e0 + j < lp) *reinterpret_cast<uint16_t *>(column + (e0 + j) * kRow) = v[j];
+                }
             }
         }
     }

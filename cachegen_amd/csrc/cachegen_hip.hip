@@ -485,7 +485,11 @@ int cg_decode_kv(const int16_t *cdf, int max_bins, const void *maxima, int max_d
         return fail(CG_ERR_ARG, "decode_kv: negative output strides, or %d token rows of one layer's keys or values "
                                 "span 4 GiB or more", kSub);
     const int64_t nsub = cg_num_subchunks(T, chunk_tokens);
-    const int block = pick_block(C, max_bins + 1);
+    // two wavefronts per block: a block's slot is held until its slowest wavefront is through
+    // its 256 symbols, and smaller blocks leave fewer finished wavefronts waiting for that
+    // (one wavefront per block loses more to the per-block set-up than it gains)
+    int block = pick_block(C, max_bins + 1);
+    if (block > 128) block = 128;
     DecodeArgs a;
     memset(&a, 0, sizeof(a));
     a.cdf = reinterpret_cast<const uint16_t *>(cdf);

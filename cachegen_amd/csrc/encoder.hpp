@@ -14,7 +14,7 @@ namespace {
 // ---- encoder (enc_new.cu:21-97, 253-307) -------------------------------------------
 // Bits are collected MSB-first in a 64-bit accumulator and leave as big-endian 32-bit words.
 // Every lane of a wavefront runs the store code whenever one lane has a word ready, so words
-// are written at fixed points, once per four symbols (per two, for byte symbols), instead of
+// are written at fixed points, once per eight symbols (per two, for byte symbols), instead of
 // whenever a lane's accumulator fills; the accumulator takes the symbols in between (a put
 // that would not fit writes a word first).
 // The E1/E2 run of a symbol is emitted at once: the n1 = clz(low ^ high) leading bits
@@ -362,14 +362,23 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
                 load_half(h);
                 // uniform; kept in a scalar register so that the loop test is scalar too
                 const int wn = __builtin_amdgcn_readfirstlane(nwords - h * 32 < 32 ? nwords - h * 32 : 32);
+                // two words = eight symbols between two visits of the store code (wn is even
+                // except in a sub-chunk's last, partial run of words)
 #pragma unroll 1
-                for (int w = 0; w < wn; ++w) {
+                for (int w = 0; w < wn; w += 2) {
                     const uint32_t v = words[w];
                     const int t = (h * 32 + w) * 4;            // first token of the word
                     if (t + 0 < id.n) enc.template put_symbol<SENTINEL, true>(v & 0xFFu);
                     if (t + 1 < id.n) enc.template put_symbol<SENTINEL, false>((v >> 8) & 0xFFu);
                     if (t + 2 < id.n) enc.template put_symbol<SENTINEL, false>((v >> 16) & 0xFFu);
                     if (t + 3 < id.n) enc.template put_symbol<SENTINEL, false>(v >> 24);
+                    if (t + 4 < id.n) {
+                        const uint32_t u = words[w + 1];       // w + 1 <= 31: wn <= 32
+                        enc.template put_symbol<SENTINEL, false>(u & 0xFFu);
+                        if (t + 5 < id.n) enc.template put_symbol<SENTINEL, false>((u >> 8) & 0xFFu);
+                        if (t + 6 < id.n) enc.template put_symbol<SENTINEL, false>((u >> 16) & 0xFFu);
+                        if (t + 7 < id.n) enc.template put_symbol<SENTINEL, false>(u >> 24);
+                    }
                     enc.w.flush_word();
                 }
             }

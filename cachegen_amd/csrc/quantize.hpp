@@ -209,7 +209,10 @@ __global__ __launch_bounds__(256) void quantize_pack_kernel(PackedQuantArgs a)
                 int64_t off;
                 if (HEADS_CONTIGUOUS) off = e;
                 else { const int h = e / a.D; off = (int64_t)h * a.sh + (e - h * a.D); }
-                regs[j][i] = *reinterpret_cast<const uint4 *>(base + j * a.st + off);
+                // read once and never again: loaded past the caches' keep-for-reuse policy
+                typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+                const u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base + j * a.st + off));
+                regs[j][i] = make_uint4(t.x, t.y, t.z, t.w);
                 m = pk_max_u16(m, regs[j][i].x & 0x7FFF7FFFu);
                 m = pk_max_u16(m, regs[j][i].y & 0x7FFF7FFFu);
                 m = pk_max_u16(m, regs[j][i].z & 0x7FFF7FFFu);

@@ -19,18 +19,6 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0
 
-# HBM bytes per launch of decode_streams_kernel measured with rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE (two runs, each scaled by what the same counter reads for a plain conversion
-# kernel of known size: x2.000 and x1.000): 292.4 MB read + 1073.7 MB written.  A profile
-# measurement of this workload, not something this script can observe while it runs.
-MEASURED_DECODE_TRAFFIC_BYTES = {"config2": 1366.1e6}
-
-# VALU wave-instructions per launch of decode_streams_kernel (rocprofv3 --pmc SQ_INSTS_VALU, same
-# profile).  The kernel's own limit is the issue of these: one per 4 cycles per SIMD for most
-# of them, 1024 SIMDs, at the clock the profile's GRBM_GUI_ACTIVE gives (2.3 GHz).
-MEASURED_DECODE_VALU_INSTS = {"config2": 378.91e6}
-VALU_ISSUE_PER_SECOND = 1024 * 2.3e9 / 4
-
 WORKLOADS = {
     # name: (layers, tokens, heads, head_size, chunk_tokens, model name for the bins table, seed)
     "config1": (2, 512, 8, 64, 512, None, 1235),
@@ -148,6 +136,145 @@ def algorithmic_bytes(L, T, C, lp, nchunks, nstreams, payload):
                 decode=2 * n + payload + side)
 
 
+def measured_counters():
+    """Per-launch counter readings of the committed rocprofv3 profiles (profiles/*.txt), kept as
+    numbers in profiles/measured_counters.json: they are measurements of a profiled run of this
+    script, not something it can observe while it runs."""
+    path = os.path.join(ROOT, "profiles", "measured_counters.json")
+    if not os.path.exists(path):
+        return {}
+    with open(path) as f:
+        return json.load(f)
+
+
+def run_workload(name, steps, warmup, fmt="vllm", copy_probe=False, keep=False):
+    """Encode + decode of one workload, timed with HIP events on the launching stream.
+    Returns a dict of figures (and, with keep=True, the tensors for further use)."""
+    import torch
+    from cachegen_amd import codec
+    from cachegen_amd.kvgen import make_kv
+
+    L, T, H, D, chunk, model, seed = WORKLOADS[name]
+    C = H * D
+    dev = torch.device("cuda:0")
+    kbins, vbins = bins_for(name, model, L)
+    kv = make_kv(L, T, H, D, seed=seed, device=dev)
+    if fmt == "huggingface":
+        kv = kv.permute(0, 1, 3, 2, 4).contiguous()
+    kb, vb = kbins.to(dev), vbins.to(dev)
+    max_bins = int(max(kbins.max(), vbins.max()))
+
+    workspace = torch.empty(codec.encode_workspace_bytes(L, T, C, chunk), dtype=torch.uint8, device=dev)
+    enc = codec.encode_kv(kv, kb, vb, chunk_tokens=chunk, max_bins=max_bins, workspace=workspace, fmt=fmt)
+    enc.check()
+    out = torch.empty_like(kv)
+
+    def encode():
+        codec.encode_kv(kv, kb, vb, chunk_tokens=chunk, max_bins=max_bins, workspace=workspace, out=enc, fmt=fmt)
+
+    def decode():
+        codec.decode_encoded(enc, kb, vb, fmt=fmt, out=out)
+
+    for _ in range(warmup):
+        encode()
+        decode()
+    torch.cuda.synchronize()
+
+    # per-phase device times: HIP events on the stream the kernels are queued on
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        ev[i][0].record()
+        encode()
+        ev[i][1].record()
+        decode()                      # a single launch of decode_streams_kernel
+        ev[i][2].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    enc_ms = sorted(e[0].elapsed_time(e[1]) for e in ev)
+    dec_ms = sorted(e[1].elapsed_time(e[2]) for e in ev)
+    enc_avg = sum(enc_ms) / len(enc_ms)
+    dec_avg = sum(dec_ms) / len(dec_ms)
+
+    if copy_probe:
+        out.copy_(kv)                 # reads and writes kv_bytes each: the known-size reference kernel
+        torch.cuda.synchronize()
+        decode()
+        torch.cuda.synchronize()
+
+    enc.check()
+    payload = enc.total_bytes()
+    nstreams = enc.lengths.numel()
+    ab = algorithmic_bytes(L, T, C, max_bins + 1, enc.num_chunks, nstreams, payload)
+    kv_bytes = ab["kv"]
+
+    # round trip must reconstruct within half a quantization step of every row
+    # (half a step plus the 16-bit rounding of the output), checked in slices of layers
+    maxq = torch.stack([kb, vb], dim=1).div(2, rounding_mode="floor").sub(1)[:, :, None, None]
+    verified = True
+    group = 8 if C <= 1024 else 4
+    for l0 in range(0, L, group):
+        xs, ys = kv[l0:l0 + group], out[l0:l0 + group]
+        if fmt == "huggingface":
+            xs, ys = xs.permute(0, 1, 3, 2, 4), ys.permute(0, 1, 3, 2, 4)
+        x = xs.reshape(-1, 2, T, C).float()
+        y = ys.reshape(-1, 2, T, C).float()
+        step = x.abs().amax(dim=-1, keepdim=True) / maxq[l0:l0 + group]
+        verified = verified and bool(((x - y).abs() <= 0.52 * step).all())
+        del x, y, step
+
+    r = {
+        "workload": "%s: %d layers x {K,V} x %d tokens x %d heads x %d, fp16, one table per %d tokens, "
+                    "AR(1) rho=0.9 lognormal-channel generator seed %d%s"
+                    % (name, L, T, H, D, chunk, seed, "" if fmt == "vllm" else ", layout [L,2,H,T,D]"),
+        "kv_bytes": kv_bytes, "streams": nstreams, "wall_ms_per_step": wall * 1000.0 / steps,
+        "encode_ms": enc_avg, "decode_ms": dec_avg,
+        "encode_ms_median": enc_ms[len(enc_ms) // 2], "decode_ms_median": dec_ms[len(dec_ms) // 2],
+        "encode_GBps": kv_bytes / (enc_avg * 1e-3) / 1e9, "decode_GBps": kv_bytes / (dec_avg * 1e-3) / 1e9,
+        "encode_roofline_frac": ab["encode"] / (enc_avg * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+        "decode_roofline_frac": ab["decode"] / (dec_avg * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+        "compression_ratio_payload": kv_bytes / payload,
+        "compression_ratio_total": kv_bytes / (payload + ab["side"]),
+        "payload_bytes": payload, "algorithmic_bytes": ab, "round_trip_within_half_step": verified,
+    }
+    if chunk > 256:
+        # streaming case: latency of decoding one chunk on its own
+        tdim = 2 if fmt == "vllm" else 3
+        one = codec.encode_kv(kv.narrow(tdim, 0, chunk), kb, vb, chunk_tokens=chunk, max_bins=max_bins, fmt=fmt)
+        one_out = torch.empty_like(kv.narrow(tdim, 0, chunk))
+        for _ in range(3):
+            codec.decode_encoded(one, kb, vb, fmt=fmt, out=one_out)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(10):
+            codec.decode_encoded(one, kb, vb, fmt=fmt, out=one_out)
+        e1.record()
+        torch.cuda.synchronize()
+        r["decode_ms_per_%d_token_chunk" % chunk] = e0.elapsed_time(e1) / 10
+        del one, one_out
+    if keep:
+        r["_keep"] = dict(kv=kv, enc=enc, kbins=kbins, vbins=vbins, chunk=chunk, L=L, T=T, C=C)
+    else:
+        del kv, out, enc, workspace
+        torch.cuda.empty_cache()
+    return r
+
+
+def other_config_summary(r):
+    """The figures of a secondary workload that go into the main JSON line."""
+    keys = ["encode_ms", "decode_ms", "encode_GBps", "decode_GBps", "encode_roofline_frac", "decode_roofline_frac",
+            "compression_ratio_payload", "compression_ratio_total", "round_trip_within_half_step"]
+    out = {"workload": r["workload"]}
+    for k in keys:
+        out[k] = round(r[k], 4) if isinstance(r[k], float) else r[k]
+    for k in r:
+        if k.startswith("decode_ms_per_"):
+            out[k] = round(r[k], 4)
+    return out
+
+
 def cpu_baseline(kv_cpu, kbins, vbins, chunk, sample_tokens):
     """The oracle's CPU path (C, OpenMP over streams) on the first `sample_tokens` tokens."""
     import numpy as np
@@ -190,6 +317,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="config2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="skip the short runs of configs 3, 4 and 5 that the default workload appends")
     ap.add_argument("--cpu-sample-tokens", type=int, default=8192)
     ap.add_argument("--fmt", default="vllm", choices=["vllm", "huggingface"],
                     help="layout of the KV tensor: [L,2,T,H,D] (vllm, the metric's layout) or [L,2,H,T,D]")
@@ -206,81 +335,15 @@ def main():
         return
 
     import torch
-    from cachegen_amd import codec
-    from cachegen_amd.kvgen import make_kv
-
-    L, T, H, D, chunk, model, seed = WORKLOADS[args.workload]
-    C = H * D
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-    kbins, vbins = bins_for(args.workload, model, L)
-    kv = make_kv(L, T, H, D, seed=seed, device=dev)
+    torch.cuda.set_device(0)
     fmt = args.fmt
-    if fmt == "huggingface":
-        kv = kv.permute(0, 1, 3, 2, 4).contiguous()
-    kb, vb = kbins.to(dev), vbins.to(dev)
-    max_bins = int(max(kbins.max(), vbins.max()))
-
-    workspace = torch.empty(codec.encode_workspace_bytes(L, T, C, chunk), dtype=torch.uint8, device=dev)
-    enc = codec.encode_kv(kv, kb, vb, chunk_tokens=chunk, max_bins=max_bins, workspace=workspace, fmt=fmt)
-    enc.check()
-    out = torch.empty_like(kv)
-
-    def encode():
-        codec.encode_kv(kv, kb, vb, chunk_tokens=chunk, max_bins=max_bins, workspace=workspace, out=enc, fmt=fmt)
-
-    def decode():
-        codec.decode_encoded(enc, kb, vb, fmt=fmt, out=out)
-
-    for _ in range(args.warmup):
-        encode()
-        decode()
-    torch.cuda.synchronize()
-
-    # per-phase device times: HIP events on the stream the kernels are queued on
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        ev[i][0].record()
-        encode()
-        ev[i][1].record()
-        decode()                      # a single launch of decode_streams_kernel
-        ev[i][2].record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-
-    enc_ms = sorted(e[0].elapsed_time(e[1]) for e in ev)
-    dec_ms = sorted(e[1].elapsed_time(e[2]) for e in ev)
-    enc_avg = sum(enc_ms) / len(enc_ms)
-    dec_avg = sum(dec_ms) / len(dec_ms)
-    ms_per_step = wall * 1000.0 / args.steps
-
-    if args.copy_probe:
-        out.copy_(kv)                 # reads and writes kv_bytes each: the known-size reference kernel
-        torch.cuda.synchronize()
-        decode()
-        torch.cuda.synchronize()
-
-    enc.check()
-    payload = enc.total_bytes()
-    nstreams = enc.lengths.numel()
-    ab = algorithmic_bytes(L, T, C, max_bins + 1, enc.num_chunks, nstreams, payload)
-    kv_bytes = ab["kv"]
-
-    # round trip must reconstruct within half a quantization step of every row
-    # (half a step plus the 16-bit rounding of the output), checked in slices of layers
-    maxq = torch.stack([kb, vb], dim=1).div(2, rounding_mode="floor").sub(1)[:, :, None, None]
-    verified = True
-    for l0 in range(0, L, 8):
-        xs, ys = kv[l0:l0 + 8], out[l0:l0 + 8]
-        if fmt == "huggingface":
-            xs, ys = xs.permute(0, 1, 3, 2, 4), ys.permute(0, 1, 3, 2, 4)
-        x = xs.reshape(-1, 2, T, C).float()
-        y = ys.reshape(-1, 2, T, C).float()
-        step = x.abs().amax(dim=-1, keepdim=True) / maxq[l0:l0 + 8]
-        verified = verified and bool(((x - y).abs() <= 0.52 * step).all())
-        del x, y
+    r = run_workload(args.workload, args.steps, args.warmup, fmt=fmt, copy_probe=args.copy_probe, keep=True)
+    kept = r.pop("_keep")
+    ab = r["algorithmic_bytes"]
+    kv_bytes = r["kv_bytes"]
+    ms_per_step = r["wall_ms_per_step"]
+    counters = measured_counters().get(args.workload, {}).get("decode_streams_kernel", {})
+    traffic = counters.get("fetch_bytes", 0) + counters.get("write_bytes", 0)
 
     result = {
         "metric": "KV encode & decode GB/s (fp16 input) + % HBM roofline + compression ratio",
@@ -296,73 +359,76 @@ def main():
         "dtype": "u32",
         "data": "synthetic",
         "config": {
-            "workload": "%s: %d layers x {K,V} x %d tokens x %d heads x %d, fp16, one table per %d tokens, "
-                        "AR(1) rho=0.9 lognormal-channel generator seed %d%s"
-                        % (args.workload, L, T, H, D, chunk, seed, "" if fmt == "vllm" else ", layout [L,2,H,T,D]"),
+            "workload": r["workload"],
             "value_is": "fp16 KV bytes encoded plus decoded per second of a full encode+decode step",
             "kv_bytes": kv_bytes,
-            "streams": nstreams,
+            "streams": r["streams"],
         },
-        "encode_GBps": round(kv_bytes / (enc_avg * 1e-3) / 1e9, 3),
-        "decode_GBps": round(kv_bytes / (dec_avg * 1e-3) / 1e9, 3),
-        "encode_ms": round(enc_avg, 4),
-        "decode_ms": round(dec_avg, 4),
-        "encode_ms_median": round(enc_ms[len(enc_ms) // 2], 4),
-        "decode_ms_median": round(dec_ms[len(dec_ms) // 2], 4),
-        "encode_roofline_frac": round(ab["encode"] / (enc_avg * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
-        "decode_roofline_frac": round(ab["decode"] / (dec_avg * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
-        "compression_ratio_payload": round(kv_bytes / payload, 3),
-        "compression_ratio_total": round(kv_bytes / (payload + ab["side"]), 3),
-        "payload_bytes": payload,
-        "round_trip_within_half_step": verified,
+        "encode_GBps": round(r["encode_GBps"], 3),
+        "decode_GBps": round(r["decode_GBps"], 3),
+        "encode_ms": round(r["encode_ms"], 4),
+        "decode_ms": round(r["decode_ms"], 4),
+        "encode_ms_median": round(r["encode_ms_median"], 4),
+        "decode_ms_median": round(r["decode_ms_median"], 4),
+        "encode_roofline_frac": round(r["encode_roofline_frac"], 4),
+        "decode_roofline_frac": round(r["decode_roofline_frac"], 4),
+        "compression_ratio_payload": round(r["compression_ratio_payload"], 3),
+        "compression_ratio_total": round(r["compression_ratio_total"], 3),
+        "payload_bytes": r["payload_bytes"],
+        "round_trip_within_half_step": r["round_trip_within_half_step"],
         "roofline": {
             "kernel": "decode_streams_kernel",
             "bound": "hbm",
-            "achieved": round(ab["decode"] / (dec_avg * 1e-3) / 1e9, 2),
+            "achieved": round(ab["decode"] / (r["decode_ms"] * 1e-3) / 1e9, 2),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
-            "frac": round(ab["decode"] / (dec_avg * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
-            "traffic": MEASURED_DECODE_TRAFFIC_BYTES.get(args.workload),
+            "frac": round(r["decode_roofline_frac"], 4),
+            "traffic": traffic if traffic else None,       # profiles/measured_counters.json; null = not profiled
             "algorithmic_bytes": ab["decode"],
-            "avg_launch_ms": round(dec_avg, 4),
+            "avg_launch_ms": round(r["decode_ms"], 4),
         },
     }
-    if args.workload in MEASURED_DECODE_VALU_INSTS:
-        insts = MEASURED_DECODE_VALU_INSTS[args.workload]
+    if "valu_insts" in counters:
+        # The kernel's own limit is the issue of vector instructions: one per 4 cycles per SIMD for
+        # most of them, 1024 SIMDs, at the clock the profile's GRBM_GUI_ACTIVE gives (2.3 GHz).
+        insts = counters["valu_insts"]
         result["valu_issue"] = {
             "kernel": "decode_streams_kernel",
             "insts_per_launch": insts,
             "insts_per_symbol_and_lane": round(insts * 64 / (kv_bytes / 2), 1),
-            "frac_of_issue_rate": round(insts / (dec_avg * 1e-3) / VALU_ISSUE_PER_SECOND, 3),
+            "frac_of_issue_rate": round(insts / (r["decode_ms"] * 1e-3) / (1024 * 2.3e9 / 4), 3),
             "note": "profile counter x live duration; above 1 where cheap instructions issue in under 4 cycles",
         }
+    for k in r:
+        if k.startswith("decode_ms_per_"):
+            result[k] = round(r[k], 4)
     # what one chunk weighs on the wire in the two flat containers (first chunk, vllm layout only)
     if fmt == "vllm":
         from cachegen_amd.serde import wire
+        enc = kept["enc"]
         flat_blob = wire.pack_chunks(enc, 0, 1)[0]
         compact_blob = wire.pack_chunks(enc, 0, 1, compact=True)[0]
-        chunk_fp16 = 2 * L * min(chunk, T) * C * 2
+        chunk_fp16 = 2 * kept["L"] * min(kept["chunk"], kept["T"]) * kept["C"] * 2
         result["first_chunk_container"] = {
             "fp16_bytes": chunk_fp16, "flat_bytes": len(flat_blob), "compact_bytes": len(compact_blob),
             "ratio_flat": round(chunk_fp16 / len(flat_blob), 3), "ratio_compact": round(chunk_fp16 / len(compact_blob), 3)}
-    if chunk > 256:
-        # streaming case: latency of decoding one chunk on its own
-        tdim = 2 if fmt == "vllm" else 3
-        one = codec.encode_kv(kv.narrow(tdim, 0, chunk), kb, vb, chunk_tokens=chunk, max_bins=max_bins, fmt=fmt)
-        one_out = torch.empty_like(kv.narrow(tdim, 0, chunk))
-        for _ in range(3):
-            codec.decode_encoded(one, kb, vb, fmt=fmt, out=one_out)
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(10):
-            codec.decode_encoded(one, kb, vb, fmt=fmt, out=one_out)
-        e1.record()
-        torch.cuda.synchronize()
-        result["decode_ms_per_%d_token_chunk" % chunk] = round(e0.elapsed_time(e1) / 10, 4)
     if not args.no_cpu_baseline:
+        kv = kept["kv"]
         kv_vllm = kv if fmt == "vllm" else kv.permute(0, 1, 3, 2, 4)
-        result["cpu_baseline"] = cpu_baseline(kv_vllm[:, :, :args.cpu_sample_tokens].cpu(), kbins, vbins, chunk,
-                                              args.cpu_sample_tokens)
+        result["cpu_baseline"] = cpu_baseline(kv_vllm[:, :, :args.cpu_sample_tokens].cpu(), kept["kbins"], kept["vbins"],
+                                              kept["chunk"], args.cpu_sample_tokens)
+    del kept
+    torch.cuda.empty_cache()
+    if args.workload == "config2" and fmt == "vllm" and not args.no_other_configs:
+        # the other benchmark configurations, a few steps each, so that their figures are observed
+        # by whoever runs this script and not only quoted
+        others = {}
+        for name in ("config3", "config4"):
+            others[name] = other_config_summary(run_workload(name, max(2, min(args.steps, 5)), 1))
+        lv = run_levels(argparse.Namespace(steps=max(2, min(args.steps, 5)), warmup=1), quiet=True)
+        others["config5"] = {k: lv[k] for k in ("config", "encode_four_levels_at_once_ms", "encode_four_levels_separately_ms",
+                                                "encode_at_once_GBps_per_level", "decode_four_levels_ms", "levels")}
+        result["other_configs"] = others
     print(json.dumps(result))
 
 

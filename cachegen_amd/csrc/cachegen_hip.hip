@@ -304,13 +304,13 @@ struct LevelOut {
 // Tables, streams and payload of one level from its symbols (packed words `sym4`, or byte
 // symbols [2L, T, C]): calculate_cdf + encode_fast_new + collect_bytes for every chunk
 // (encoder.py:265-292, 209-222).
+// The level's status word has been set to zero by an earlier launch of the same call.
 int code_and_compact(const LevelOut &o, const uint32_t *sym4, const uint8_t *sym_bytes, const EncodeWorkspace &w,
                      int64_t L, int64_t T, int64_t C, int64_t chunk_tokens, hipStream_t s)
 {
     const int64_t rows = 2 * L;
     const int lp = o.max_bins + 1;
     uint16_t *tables = reinterpret_cast<uint16_t *>(o.cdf);
-    clear_status_kernel<<<1, 1, 0, s>>>(o.status);
 
     const int block = pick_block(C, lp);
     EncodeArgs a;
@@ -409,9 +409,10 @@ int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int
     if (packed) {
         uint32_t *sym4 = reinterpret_cast<uint32_t *>(w.symbols);
         if (int rc = launch_quantize_pack(kv, kv_dt, L, T, H, D, sl, skv, st, sh, key_bins, value_bins, sym4,
-                                          maxima, w.nsub, chunk_tokens, delta_group, s)) return rc;
+                                          maxima, w.nsub, chunk_tokens, delta_group, s, status)) return rc;
         return code_and_compact(o, sym4, nullptr, w, L, T, C, chunk_tokens, s);
     }
+    clear_status_kernel<<<1, 1, 0, s>>>(status);
     if (int rc = launch_quantize(kv, kv_dt, L, T, H, D, sl, skv, st, sh, key_bins, value_bins, w.symbols, maxima, s)) return rc;
     return code_and_compact(o, nullptr, w.symbols, w, L, T, C, chunk_tokens, s);
 }
@@ -446,7 +447,7 @@ int cg_encode_kv_levels(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t
         // symbols written once per level
         uint32_t *sym4 = reinterpret_cast<uint32_t *>(w.symbols);
         if (int rc = launch_quantize_pack(kv, kv_dt, L, T, H, D, sl, skv, st, sh, nullptr, nullptr, sym4, maxima,
-                                          w.nsub, chunk_tokens, 0, s, nlevels, key_bins, value_bins,
+                                          w.nsub, chunk_tokens, 0, s, status, nlevels, key_bins, value_bins,
                                           (int64_t)(w.symbols_bytes / 4))) return rc;
     }
     for (int v = 0; v < nlevels; ++v) {
@@ -457,6 +458,7 @@ int cg_encode_kv_levels(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t
             if (int rc = code_and_compact(o, reinterpret_cast<uint32_t *>(symbols), nullptr, w, L, T, C, chunk_tokens, s)) return rc;
         } else {
             // shapes the vector loads cannot take: one plain quantization pass per level
+            clear_status_kernel<<<1, 1, 0, s>>>(status + v);
             if (int rc = launch_quantize(kv, kv_dt, L, T, H, D, sl, skv, st, sh, key_bins[v], value_bins[v], symbols, maxima, s)) return rc;
             if (int rc = code_and_compact(o, nullptr, symbols, w, L, T, C, chunk_tokens, s)) return rc;
         }

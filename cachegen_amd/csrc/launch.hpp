@@ -82,6 +82,11 @@ int launch_scan(const int32_t *lengths, int64_t n, int32_t clamp, int64_t *offse
 {
     const int64_t ntiles = ceil_div(n, kScanTile);
     int64_t *sums = static_cast<int64_t *>(scratch);
+    if (ntiles > 1 && n <= kScanSmallMax) {
+        // a few thousand values: one block does it all, two launches fewer
+        scan_small_kernel<<<dim3(1), dim3(kScanSmallThreads), 0, stream>>>(lengths, (int32_t)n, clamp, offsets);
+        return check_launch("scan_lengths");
+    }
     if (ntiles == 1) {
         scan_apply_kernel<<<dim3(1), dim3(kScanThreads), 0, stream>>>(lengths, n, clamp, nullptr, offsets);
         return check_launch("scan_lengths");
@@ -168,12 +173,15 @@ void launch_quantize_pack_nu(const PackedQuantArgs &a, int64_t nblocks, hipStrea
 int launch_quantize_pack(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D,
                          int64_t sl, int64_t skv, int64_t st, int64_t sh, const float *key_bins,
                          const float *value_bins, uint32_t *sym4, void *maxima, int64_t nsub,
-                         int64_t S, int delta_group, hipStream_t stream, int nlevels = 0,
+                         int64_t S, int delta_group, hipStream_t stream, int32_t *status, int nlevels = 0,
                          const float *const *key_bins_lv = nullptr, const float *const *value_bins_lv = nullptr,
                          int64_t level_words = 0)
 {
     PackedQuantArgs a;
     memset(&a, 0, sizeof(a));
+    // status: one word per level (one word when nlevels == 0), consecutive
+    a.nstatus = nlevels > 0 ? nlevels : 1;
+    for (int v = 0; v < a.nstatus; ++v) a.status[v] = status + v;
     a.nlevels = nlevels;
     for (int v = 0; v < nlevels; ++v) {
         a.key_bins_lv[v] = key_bins_lv[v];

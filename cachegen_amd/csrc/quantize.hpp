@@ -163,6 +163,10 @@ struct PackedQuantArgs {
     int32_t nlevels;
     const float *key_bins_lv[kMaxLevels], *value_bins_lv[kMaxLevels];
     int64_t level_words;
+    // status words of the encode call (one per level) that this launch, the first of the call,
+    // sets to zero
+    int32_t nstatus;
+    int32_t *status[kMaxLevels];
     uint32_t *sym4;
     uint16_t *maxima;       // [2L, T]
     int32_t nunits;         // C / 8
@@ -177,9 +181,15 @@ struct PackedQuantArgs {
 // MULTI: the rows are loaded and their maxima found once, then quantized at each of
 // a.nlevels levels (the adaptive-streaming use: run_adaptation.py:63-72 encodes every chunk
 // at QUANT_LEVEL 1..3); the maxima do not depend on the level.
+__device__ __forceinline__ void clear_statuses(const PackedQuantArgs &a)
+{
+    if (blockIdx.x == 0 && threadIdx.x < a.nstatus) *a.status[threadIdx.x] = 0;
+}
+
 template <int DT, bool HEADS_CONTIGUOUS, int NU, bool MULTI = false>
 __global__ __launch_bounds__(256) void quantize_pack_kernel(PackedQuantArgs a)
 {
+    clear_statuses(a);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     int64_t b = blockIdx.x;
     const int tq = (int)(b & 15) * 4 + wave;      // word index inside the sub-chunk slot
@@ -273,6 +283,7 @@ __global__ __launch_bounds__(256) void quantize_pack_kernel(PackedQuantArgs a)
 template <int DT, bool HEADS_CONTIGUOUS, int NU>
 __global__ __launch_bounds__(256) void quantize_pack_delta_kernel(PackedQuantArgs a)
 {
+    clear_statuses(a);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     int64_t b = blockIdx.x;
     const int tq = (int)(b & 15) * 4 + wave;

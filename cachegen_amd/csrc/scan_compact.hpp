@@ -110,6 +110,51 @@ __global__ __launch_bounds__(kScanThreads) void scan_apply_kernel(
     }
 }
 
+// The whole running sum in one launch of one block, for up to kScanSmallMax values (the byte
+// counts of the encoder's tiles): every thread owns up to 16 consecutive values, the block scans
+// the 1024 thread totals with wavefront shuffles, and every thread writes its run.
+constexpr int kScanSmallThreads = 1024;
+constexpr int kScanSmallPer = 16;
+constexpr int kScanSmallMax = kScanSmallThreads * kScanSmallPer;
+
+__global__ __launch_bounds__(kScanSmallThreads) void scan_small_kernel(
+    const int32_t *__restrict__ lengths, int32_t n, int32_t clamp, int64_t *__restrict__ offsets)
+{
+    __shared__ int64_t wave_totals[kScanSmallThreads / 64];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int per = (n + kScanSmallThreads - 1) / kScanSmallThreads;      // <= kScanSmallPer
+    const int lo = tid * per;
+    int32_t v[kScanSmallPer];
+    int64_t mine = 0;
+#pragma unroll
+    for (int j = 0; j < kScanSmallPer; ++j) {
+        int32_t x = (j < per && lo + j < n) ? lengths[lo + j] : 0;
+        x = x < 0 ? 0 : (x > clamp ? clamp : x);
+        v[j] = x;
+        mine += x;
+    }
+    // inclusive running sum over the wavefront, then over the 16 wavefront totals
+    int64_t incl = mine;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const int64_t up = __shfl_up(incl, o, 64);
+        if (lane >= o) incl += up;
+    }
+    if (lane == 63) wave_totals[wave] = incl;
+    __syncthreads();
+    int64_t before = 0;
+    for (int w = 0; w < wave; ++w) before += wave_totals[w];
+    int64_t run = before + incl - mine;
+#pragma unroll
+    for (int j = 0; j < kScanSmallPer; ++j) {
+        if (j < per && lo + j < n) {
+            offsets[lo + j] = run;
+            run += v[j];
+            if (lo + j == n - 1) offsets[n] = run;
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------------
 // collect_bytes (encoder.py:209-222).  A block owns 256 consecutive streams, i.e. one
 // contiguous range of the payload, and assembles it in LDS, 16 KiB at a time: every thread

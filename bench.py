@@ -399,6 +399,12 @@ def main():
             "frac_of_issue_rate": round(insts / (r["decode_ms"] * 1e-3) / (1024 * 2.3e9 / 4), 3),
             "note": "profile counter x live duration; above 1 where cheap instructions issue in under 4 cycles",
         }
+    enc_counters = measured_counters().get(args.workload, {}).get("encode_all_kernels")
+    if enc_counters:
+        result["encode_traffic"] = {
+            "bytes": enc_counters["fetch_bytes"] + enc_counters["write_bytes"], "algorithmic_bytes": ab["encode"],
+            "ratio": round((enc_counters["fetch_bytes"] + enc_counters["write_bytes"]) / ab["encode"], 2),
+            "source": enc_counters["source"]}
     for k in r:
         if k.startswith("decode_ms_per_"):
             result[k] = round(r[k], 4)

@@ -260,8 +260,10 @@ __global__ __launch_bounds__(256) void quantize_pack_kernel(PackedQuantArgs a)
                         const uint32_t bits = (k & 1) ? (src >> 16) : (src & 0xFFFFu);
                         const float v = load16f<DT>(bits);
                         const float s = __fadd_rn(__fmul_rn(v, factor[j]), maxq);
-                        const float r = fmaxf(__builtin_rintf(s), 0.0f);     // NaN -> 0
-                        w = __builtin_amdgcn_cvt_pk_u8_f32(r, (uint32_t)j, w);
+                        // the conversion itself rounds to nearest even, turns a NaN (0 * inf of an
+                        // all-zero row) and anything negative into 0 and saturates at 255: the
+                        // round-half-even, int8 cast and NaN rule of encoder.py:56-57 in one step
+                        w = __builtin_amdgcn_cvt_pk_u8_f32(s, (uint32_t)j, w);
                     }
                     words[k] = w;
                 }

@@ -169,6 +169,36 @@ def test_nan_and_infinite_rows_match_oracle(oracle):
             assert nan_ref.any() and np.array_equal(got[~nan_ref], ref[~nan_ref]), (dtype, out_dtype)
 
 
+def test_ties_round_to_even_in_the_fused_quantizer(oracle):
+    """Rows made of halves and quarters of the row maximum, so that x * (MAX / max) + MAX lands
+    exactly on .5 for many elements (0.5 * 15 + 15 = 22.5 -> 22, -0.5 * 7 + 7 = 3.5 -> 4, ...):
+    the fused path rounds inside its packed float-to-byte conversion and must still round half
+    to even like torch.round (encoder.py:56-57)."""
+    codec, _ = _mods()
+    L, T, H, D = 3, 64, 2, 64
+    g = torch.Generator().manual_seed(23)
+    choices = torch.tensor([1.0, -1.0, 0.5, -0.5, 0.0, 0.25, -0.25, 0.75, -0.75, 0.125])
+    kv = choices[torch.randint(0, len(choices), (L, 2, T, H, D), generator=g)]
+    kv[..., 0] = 1.0                                             # every row's maximum is exactly 1
+    kv[1] *= 2.0                                                 # and exactly 2 in layer 1
+    kb = torch.tensor([32.0, 16.0, 12.0])
+    vb = torch.tensor([12.0, 32.0, 16.0])
+    for dtype, dt in ((torch.float16, 0), (torch.bfloat16, 1)):
+        x = kv.to(dtype)
+        flat = x.reshape(L, 2, T, H * D).contiguous().view(torch.int16).numpy().view(np.uint16)
+        want = oracle.encode_function(flat, kb.numpy(), vb.numpy(), dt)
+        wk, _ = oracle.quantize(flat[:, 0], kb.numpy(), dt)
+        assert int((wk[0] == 22).sum()) > 0 and int((wk[1] == 4).sum()) > 0      # the ties are there
+        enc = codec.encode_kv(x.to(DEV), kb, vb, chunk_tokens=T)
+        enc.check()
+        assert np.array_equal(enc.cdf[0].cpu().numpy().view(np.uint16), want["cdf"])
+        assert np.array_equal(enc.payload[:enc.total_bytes()].cpu().numpy(), want["data_chunks"][0][0])
+        lv = codec.encode_kv_levels(x.to(DEV), [(kb, vb), (vb, kb)], chunk_tokens=T)
+        assert torch.equal(lv[0].payload[:lv[0].total_bytes()], enc.payload[:enc.total_bytes()])
+        want2 = oracle.encode_function(flat, vb.numpy(), kb.numpy(), dt)
+        assert np.array_equal(lv[1].payload[:lv[1].total_bytes()].cpu().numpy(), want2["data_chunks"][0][0])
+
+
 def test_rows_with_several_different_nans_keep_the_largest_pattern(oracle):
     """Two or three NaNs with different payloads and signs in one row: the stored row maximum
     is the largest sign-stripped bit pattern in the fused path, in the plain quantiser and in

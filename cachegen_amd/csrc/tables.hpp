@@ -13,8 +13,8 @@ namespace {
 
 // ------------------------------------------------------------------------------------
 // Tables (cal_cdf.cu:17-59): one lane per (chunk, row, channel) walks the chunk's tokens
-// and counts into its own LDS column hist[bin][lane] (no atomics across lanes, no bank
-// conflicts); the running sum and the normalisation
+// and counts into its own LDS column hist[bin][lane] (no lane touches another lane's
+// counter); the running sum and the normalisation
 //   cdf[i] = (uint16)((0xFFFF - max_bins) * cum[i] / cum[max_bins]) + i
 // are done per lane in 16-bit wrap-around arithmetic like the reference's uint16
 // counters, and the block writes its tables back transposed so stores coalesce.

@@ -169,6 +169,22 @@ def test_nan_and_infinite_rows_match_oracle(oracle):
             assert nan_ref.any() and np.array_equal(got[~nan_ref], ref[~nan_ref]), (dtype, out_dtype)
 
 
+@pytest.mark.parametrize("n", [1, 7, 2048, 2049, 6151, 16383, 16384, 16385, 40000, 300001])
+def test_running_sum_of_lengths_at_the_boundaries_of_its_three_forms(n):
+    """cg_scan_lengths runs as one block (up to 2048 values), as one block of 1024 threads (up
+    to 16384) or as three launches; sums are int64 and negative lengths count as zero."""
+    codec, _ = _mods()
+    g = torch.Generator().manual_seed(n)
+    lengths = torch.randint(0, 257, (n,), generator=g, dtype=torch.int32)
+    if n > 10:
+        lengths[3] = -5                                   # never produced by the encoder; counted as 0
+        lengths[n // 2] = 2_000_000_000                   # sums pass 2^31
+        lengths[n - 1] = 2_000_000_000
+    want = np.concatenate([[0], np.cumsum(np.maximum(lengths.numpy().astype(np.int64), 0))])
+    got = codec.scan_lengths(lengths.to(DEV))
+    assert got.dtype == torch.int64 and np.array_equal(got.cpu().numpy(), want)
+
+
 def test_ties_round_to_even_in_the_fused_quantizer(oracle):
     """Rows made of halves and quarters of the row maximum, so that x * (MAX / max) + MAX lands
     exactly on .5 for many elements (0.5 * 15 + 15 = 22.5 -> 22, -0.5 * 7 + 7 = 3.5 -> 4, ...):

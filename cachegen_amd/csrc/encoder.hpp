@@ -1,5 +1,5 @@
 // Part of the CacheGen KV codec library for MI355X (gfx950); included by cachegen_hip.hip, which
-// is the one translation unit.  Range encoder: bit writer, coder state, encode_streams_kernel.
+// is the one translation unit.  Range encoder: word writer, coder state, encode_streams_kernel.
 //
 // Paths in the comments are relative to LMCache/ in the reference tree:
 //   enc_new.cu = third_party/torchac_cuda/torchac_kernel_enc_new.cu
@@ -12,17 +12,23 @@
 namespace {
 
 // ---- encoder (enc_new.cu:21-97, 253-307) -------------------------------------------
-// Bits are collected MSB-first in a 64-bit accumulator and leave as big-endian 32-bit words.
-// Every lane of a wavefront runs the store code whenever one lane has a word ready, so words
-// are written at fixed points, once per eight symbols (per two, for byte symbols), instead of
-// whenever a lane's accumulator fills; the accumulator takes the symbols in between (a put
-// that would not fit writes a word first).
-// The E1/E2 run of a symbol is emitted at once: the n1 = clz(low ^ high) leading bits
-// agree, and the pending complements go in after the first of them, which in arithmetic
-// is  bits + ((2^pend - 1) << (n1 - 1))  over n1 + pend bits.  The E3 run k is the number
-// of positions below those where low has ones and high has zeros.  One combined shift by
-// n = n1 + k renormalises low and high; n <= 18 for any table whose symbols all have
-// non-zero width, because the span stays above 2^30 between symbols.
+// The reference's coder emits a bit for every E1/E2 step and counts E3 (underflow) steps as
+// pending bits that follow the next emitted bit as its complements (enc_new.cu:86-97,
+// 275-305).  That output is the binary expansion of the interval's lower end, written with
+// carries: after a total of n renormalisation steps the bits emitted or pending are the
+// lower end's first n bits, a pending run 0111..1 being a run of ones that a later carry may
+// still turn into 1000..0, and the closing `pending + 2` bits (enc_new.cu:309-317) are the
+// next two bits of the lower end plus a quarter of the window.  So the lower end is kept
+// here as one long number: its last 32 bits (`low`, the coder's window; bit 31 can differ
+// from the reference's, where an underflow step clears it, and nothing reads it) below 64
+// bits that are waiting to be written (`out`).  A symbol adds its offset to the number and
+// shifts it left by the step count n = clz(low ^ high) + (underflow steps); nothing is
+// counted or spliced per symbol.  Words leave at fixed points, once per eight symbols (every
+// lane of a wavefront runs the store code whenever one lane has a word ready); a carry out
+// of the waiting bits is added to the last word, which is therefore held back one round
+// (`cache`), and a word of all ones is only counted (`ones`) until the word after it shows
+// whether the carry comes.  n <= 18 for any table whose symbols all have non-zero width,
+// because the span stays above 2^30 between symbols.
 constexpr int kSlotTile = 256;      // streams per tile of the encoder's scratch
 
 // TILE: the stream's words go to a tile of the scratch (word w of the tile's stream t at the
@@ -30,23 +36,29 @@ constexpr int kSlotTile = 256;      // streams per tile of the encoder's scratch
 // word or byte past the stream's capacity falls outside the descriptor and is dropped by the
 // hardware, so nothing is compared or counted per word.
 template <bool ALIGNED, bool TILE = false>
-struct BitWriter {
+struct WordWriter {
     uint8_t *wptr;          // where the next word goes
     int wstride;            // bytes from one word of the stream to the next (4: contiguous)
     int cap;
-    int nbytes;
+    int nbytes;             // bytes written so far; -4 before the held-back word's first, empty turn
     __amdgpu_buffer_rsrc_t tile;    // TILE: the block's tile
     uint32_t voff, voff0;           // TILE: byte offset in the tile of the next word, and of the first
-    uint64_t acc;           // the low 64 - room bits are waiting to be written; bits above are stale
-    // free bits of the accumulator: counted this way, the subtraction that books a put borrows
-    // exactly when the bits do not fit, and that borrow is the test
-    uint32_t room;
 
-    // the last words of a stream that does not fit its slot: keep what fits
-    __device__ __forceinline__ void store_clipped(uint32_t word)
+    __device__ __forceinline__ void init(uint8_t *dst, int stride, int capacity)
     {
-        for (int j = 0; j < 4; ++j)
-            if (nbytes + j < cap) wptr[j] = (uint8_t)(word >> (24 - 8 * j));
+        // the first word stored is the empty held-back word: it goes one word before the
+        // stream (TILE: the offset wraps and the hardware drops the store)
+        wptr = dst - stride;
+        wstride = stride;
+        cap = capacity;
+        nbytes = -4;
+        voff = voff0 = 0;
+    }
+    __device__ __forceinline__ void init_tile(__amdgpu_buffer_rsrc_t rsrc, uint32_t first)
+    {
+        tile = rsrc;
+        voff0 = first;
+        voff = first - kSlotTile * 4;
     }
 
     __device__ __forceinline__ void store_word(uint32_t word)
@@ -56,121 +68,180 @@ struct BitWriter {
             voff += kSlotTile * 4;
             return;
         }
-        if (__builtin_expect(nbytes + 4 <= cap, 1)) {
-            if (ALIGNED) {
-                *reinterpret_cast<uint32_t *>(wptr) = __builtin_bswap32(word);
+        if (nbytes >= 0) {
+            if (__builtin_expect(nbytes + 4 <= cap, 1)) {
+                if (ALIGNED) {
+                    *reinterpret_cast<uint32_t *>(wptr) = __builtin_bswap32(word);
+                } else {
+                    wptr[0] = (uint8_t)(word >> 24);
+                    wptr[1] = (uint8_t)(word >> 16);
+                    wptr[2] = (uint8_t)(word >> 8);
+                    wptr[3] = (uint8_t)word;
+                }
             } else {
-                wptr[0] = (uint8_t)(word >> 24);
-                wptr[1] = (uint8_t)(word >> 16);
-                wptr[2] = (uint8_t)(word >> 8);
-                wptr[3] = (uint8_t)word;
+                // the last words of a stream that does not fit its slot: keep what fits
+                for (int j = 0; j < 4; ++j)
+                    if (nbytes + j < cap) wptr[j] = (uint8_t)(word >> (24 - 8 * j));
             }
-        } else {
-            store_clipped(word);
         }
         wptr += wstride;
         nbytes += 4;
     }
 
-    // write one word if 32 bits are waiting
-    __device__ __forceinline__ void flush_word()
+    // the stream's last `nbits` bits (fewer than 32, left-aligned in `word`), byte by byte
+    // (enc_new.cu:42-55); returns the stream length
+    __device__ __forceinline__ int finish(uint32_t word, int nbits)
     {
-        if (room <= 32u) {
-            store_word((uint32_t)(acc >> (32u - room)));
-            room += 32u;
-        }
-    }
-
-    // append the low m bits of v (v < 2^m), 0 <= m <= 32 (m = 0 needs v = 0).  ROOM: the caller
-    // knows that at most 32 bits are waiting (it has just called flush_word), so they fit.
-    // `more` (default 0): a second addend, for callers whose value is a sum of two parts that
-    // together stay below 2^m; the freshly shifted accumulator has m zero bits at the bottom, so
-    // the parts are added in (one three-operand add) instead of summed and then or-ed in
-    template <bool ROOM = false>
-    __device__ __forceinline__ void put(uint32_t v, int m, uint32_t more = 0)
-    {
-        uint32_t left;
-        if (__builtin_expect(__builtin_usub_overflow(room, (uint32_t)m, &left), 0) && !ROOM) {
-            flush_word();                                  // more than 32 bits were waiting
-            left = room - (uint32_t)m;
-        }
-        room = left;
-        acc <<= m;
-        acc = (acc & 0xFFFFFFFF00000000ull) | (uint32_t)((uint32_t)acc + v + more);
-    }
-
-    // one bit, then `count` copies of its complement (any count): the general form of
-    // append_bit_and_pending (enc_new.cu:86-97); not on the common path
-    __device__ __forceinline__ void bit_and_run(uint32_t bit, uint32_t count)
-    {
-        uint32_t pv = bit;
-        int pm = 1;
-        for (;;) {
-            put(pv, pm);
-            flush_word();
-            if (count == 0) break;
-            pm = count < 32u ? (int)count : 32;
-            pv = bit ? 0u : (pm == 32 ? 0xFFFFFFFFu : ((1u << pm) - 1u));
-            count -= (uint32_t)pm;
-        }
-    }
-
-    // write what is left, the last partial word byte by byte (enc_new.cu:42-55); returns
-    // the stream length
-    __device__ __forceinline__ int finish()
-    {
-        flush_word();
-        flush_word();
-        const int nacc = 64 - (int)room;
         if (TILE) nbytes = (int)((voff - voff0) / kSlotTile);     // four bytes per word written
-        if (nacc > 0) {
-            uint32_t r = (uint32_t)(acc << (32 - nacc));
-            for (int left = nacc, j = 0; left > 0; left -= 8, ++j) {
-                if (TILE) __builtin_amdgcn_raw_buffer_store_b8((char)(r >> 24), tile, (int)(voff + j), 0, 0);
-                else if (nbytes < cap) wptr[j] = (uint8_t)(r >> 24);
-                nbytes++;
-                r <<= 8;
-            }
+        for (int left = nbits, j = 0; left > 0; left -= 8, ++j) {
+            if (TILE) __builtin_amdgcn_raw_buffer_store_b8((char)(word >> 24), tile, (int)(voff + j), 0, 0);
+            else if (nbytes < cap) wptr[j] = (uint8_t)(word >> 24);
+            nbytes++;
+            word <<= 8;
         }
         return nbytes;
     }
 };
 
-// The coder state is (low, span) with span = high - low + 1 held modulo 2^32: 0 stands for
-// the full range 2^32 (the initial state, and any later interval that is exactly a binary
-// fraction), where floor(span * c / 2^16) is simply c << 16.  Renormalising by n bits maps
-// span to span << n for E1/E2 and E3 steps alike.
+// The coder state is the number described above plus the interval's width `span`, held
+// modulo 2^32: 0 stands for the full range 2^32 (the initial state, and any later interval
+// that is exactly a binary fraction), where floor(span * c / 2^16) is simply c << 16.
+// Renormalising by n bits maps span to span << n for E1/E2 and E3 steps alike.
 template <int BS, bool ALIGNED, bool TILE = false>
 struct RangeEncoder {
     lds_char *col;          // this lane's table column: entry e at byte e * 2 * TableStride<BS>::k16
     uint32_t smax;          // lp - 2: the largest symbol
-    uint32_t low, span, pend;
+    uint32_t span;
+    // the number's last 96 bits: `tail` holds the window (its lower half, called low in the
+    // comments) and above it the first 32 of the bits waiting to be written, `out_hi` the rest
+    // of them: 63 - room bits wait, and above them there may be a carry (0 or 1) that belongs
+    // to the held-back word
+    uint64_t tail;
+    uint32_t out_hi;
+    // counted this way, the subtraction that books a shift borrows exactly when the bits (and
+    // the place for a carry above them) do not fit, and that borrow is the test
+    uint32_t room;
+    uint32_t cache;         // the last complete word, not yet written: a carry may still reach it
+    uint32_t ones;          // words of all ones that follow it
+    uint32_t plain;         // 0xFFFFFFFF while `ones` is 0, else 0: a word below it is stored the short way
     // the coded symbol's two table entries, each shifted left by 16: only ever written by
     // loads into the upper half, so that the lower halves stay zero
     uint32_t bound_lo, bound_hi;
-    BitWriter<ALIGNED, TILE> w;
+    WordWriter<ALIGNED, TILE> w;
 
-    __device__ __forceinline__ void init(const uint16_t *column, int lp, uint8_t *dst, int wstride, int cap)
+    __device__ __forceinline__ void init(const uint16_t *column, int lp)
     {
         col = (lds_char *)column;
         bound_lo = 0;
         bound_hi = 0;
         smax = (uint32_t)(lp - 2);
-        low = 0;
         span = 0;
-        pend = 0;
-        w.wptr = dst;
-        w.wstride = wstride;
-        w.cap = cap;
-        w.nbytes = 0;
-        w.voff = w.voff0 = 0;
-        w.acc = 0;
-        w.room = 64;
+        tail = 0;
+        out_hi = 0;
+        room = 63;
+        cache = 0;
+        ones = 0;
+        plain = 0xFFFFFFFFu;
+    }
+
+    // the held-back word, raised by the carry, and the words of all ones behind it (which the
+    // carry turns into zeros); not on the common path
+    __device__ __forceinline__ void release(uint32_t carry)
+    {
+        w.store_word(cache + carry);
+        for (; ones; --ones) w.store_word(carry ? 0u : 0xFFFFFFFFu);
+        plain = 0xFFFFFFFFu;
+    }
+
+    // takes the top 32 waiting bits (and the carry above them); needs at least 32 waiting
+    __device__ __forceinline__ void flush_word()
+    {
+        const uint32_t sh = 31u - room;                 // waiting bits that stay
+        const uint32_t out_lo = (uint32_t)(tail >> 32);
+        const uint64_t top = (((uint64_t)out_hi << 32) | out_lo) >> sh;
+        const uint32_t word = (uint32_t)top, carry = (uint32_t)(top >> 32);
+        tail = ((uint64_t)__builtin_amdgcn_ubfe(out_lo, 0u, sh) << 32) | (uint32_t)tail;
+        out_hi = 0;
+        room += 32u;
+        if (__builtin_expect(word < plain, 1)) {
+            w.store_word(cache + carry);
+            cache = word;
+        } else {
+            asm volatile("");
+            if (carry) {
+                release(1u);
+                cache = word;
+            } else if (word == 0xFFFFFFFFu) {
+                ones++;
+                plain = 0u;
+            } else {
+                release(0u);
+                cache = word;
+            }
+        }
+    }
+
+    // The two steps below are written out instruction by instruction, on fixed registers
+    // (tail in v[56:57], out_hi in v59, v58 as the lower half of the pair that shifts out_hi):
+    // the 96-bit add is one carry chain and the 96-bit shift two 64-bit shifts and a move, which
+    // the compiler does not find from C (it compares for the carry and shuffles the halves).
+
+    // the number grows by `add` (a carry may run into the waiting bits)
+    __device__ __forceinline__ void add_low(uint32_t add)
+    {
+        asm("v_add_co_u32 v56, vcc, v56, %2\n\t"
+            "v_addc_co_u32 v57, vcc, 0, v57, vcc\n\t"
+            "v_addc_co_u32 v59, vcc, 0, v59, vcc"
+            : "+{v[56:57]}"(tail), "+{v59}"(out_hi)
+            : "v"(add)
+            : "vcc");
+    }
+
+    // the same, then the step count of the interval [low, low + width - 1]: n1 = clz(low ^ high)
+    // E1/E2 steps and the E3 run below them, the leading zeros of (~low | high) once the first
+    // differing bit is shifted out
+    __device__ __forceinline__ int add_and_count(uint32_t add, uint32_t width)
+    {
+        int n;
+        uint32_t t;
+        asm("v_add_co_u32 v56, vcc, v56, %4\n\t"
+            "v_addc_co_u32 v57, vcc, 0, v57, vcc\n\t"
+            "v_addc_co_u32 v59, vcc, 0, v59, vcc\n\t"
+            "v_add3_u32 %1, %5, v56, -1\n\t"
+            "v_xor_b32 %0, %1, v56\n\t"
+            "v_bitop3_b32 %1, %1, v56, %1 bitop3:0xf3\n\t"
+            "v_ffbh_u32 %0, %0\n\t"
+            "v_add_lshl_u32 %1, %1, %1, %0\n\t"
+            "v_ffbh_u32 %1, %1\n\t"
+            "v_add_u32 %0, %0, %1"
+            : "=&v"(n), "=&v"(t), "+{v[56:57]}"(tail), "+{v59}"(out_hi)
+            : "v"(add), "v"(width)
+            : "vcc");
+        return n;
+    }
+
+    // the number moves left by n <= 31 bits.  ROOM: the caller knows that the bits fit
+    template <bool ROOM = false>
+    __device__ __forceinline__ void shift(int n)
+    {
+        uint32_t left;
+        if (__builtin_expect(__builtin_usub_overflow(room, (uint32_t)n, &left), 0) && !ROOM) {
+            asm volatile("");
+            flush_word();                               // more than 32 bits were waiting
+            left = room - (uint32_t)n;
+        }
+        room = left;
+        asm("v_mov_b32 v58, v57\n\t"
+            "v_lshlrev_b64 v[58:59], %2, v[58:59]\n\t"
+            "v_lshlrev_b64 v[56:57], %2, v[56:57]"
+            : "+{v[56:57]}"(tail), "+{v59}"(out_hi)
+            : "v"(n)
+            : "v58");
     }
 
     // SENTINEL: symbol smax may occur, whose upper bound is 2^16 and not the table's last
     // entry (enc_new.cu:270)
-    // FIRST: the symbol directly follows a flush_word (the first of a group)
+    // FIRST: the symbol directly follows a flush (the first of a group)
     template <bool SENTINEL, bool FIRST>
     __device__ __forceinline__ void put_symbol(uint32_t s)
     {
@@ -190,41 +261,28 @@ struct RangeEncoder {
             t_lo = bound_lo;
             width = (top ? 0u : bound_hi) - bound_lo;
         }
-        low += t_lo;
-        const uint32_t high = low + width - 1u;
-
-        const int n1 = __builtin_clz(low ^ high);       // low < high always
-        // the n1 agreed bits (none if n1 = 0) with the pending complements after the first
-        // n1 - 1 is needed below; computed as n1 + 0xFFFFFFFF its carry says whether n1 > 0
-        uint32_t n1m1;
-        const bool agreed = __builtin_uadd_overflow((uint32_t)n1, 0xFFFFFFFFu, &n1m1);
-        const uint32_t pe = agreed ? pend : 0u;
-        const int m = n1 + (int)pe;
-        if (__builtin_expect(m > 32, 0)) {
-            const uint32_t bits = low >> ((32 - n1) & 31);
-            w.bit_and_run(bits >> (n1 - 1), pe);
-            w.put(bits & ((1u << (n1 - 1)) - 1u), n1 - 1);
-        } else {
-            const uint32_t bits = __builtin_amdgcn_ubfe(low, (uint32_t)(32 - n1), (uint32_t)n1);
-            // ((1 << pe) - 1) << (n1 - 1), pe <= 31 here; with n1 = 0, pe is 0 and so is the mask
-            uint32_t fill;
-            asm("v_bfm_b32 %0, %1, %2" : "=v"(fill) : "v"(pe), "v"(n1m1));
-            w.template put<FIRST>(bits, m, fill);
-        }
-        // E3 run: leading zeros of (~low | high) below the first differing bit
-        const uint32_t z = shift_left_one_more((low & high) | ~low, n1);
-        const int k = __builtin_clz(z);
-        const int n = n1 + k;
-        pend = pend - pe + (uint32_t)k;
-        low = (low << n) & 0x7FFFFFFFu;
+        const int n = add_and_count(t_lo, width);
+        shift<FIRST>(n);
         span = width << n;
+    }
+
+    // one group of symbols is through: write a word if 32 bits are waiting
+    __device__ __forceinline__ void end_group()
+    {
+        if (room <= 31u) flush_word();
     }
 
     __device__ __forceinline__ int finish()
     {
-        pend += 1;
-        w.bit_and_run(low < 0x40000000u ? 0u : 1u, pend);
-        return w.finish();
+        // the closing bits (enc_new.cu:309-317): the two bits below `out` of the number plus a
+        // quarter of the window
+        add_low(0x40000000u);
+        shift(2);
+        end_group();
+        const uint32_t nbits = 63u - room;              // fewer than 32 are left
+        const uint32_t out_lo = (uint32_t)(tail >> 32);
+        release(out_lo >> nbits);
+        return w.finish(nbits ? out_lo << (32u - nbits) : 0u, (int)nbits);
     }
 };
 
@@ -335,15 +393,18 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
     if (TILE) {
         // the block is exactly one tile (the host launches this form only then): blockIdx.x is
         // the tile, tid the stream's place in it
-        enc.init(col, lp, nullptr, 0, a.cap);
-        enc.w.tile = __builtin_amdgcn_make_buffer_rsrc((void *)(a.out + (int64_t)blockIdx.x * ((int64_t)kSlotTile * a.cap)), 0,
-                                                       kSlotTile * a.cap, kBufferWord3);
-        enc.w.voff = enc.w.voff0 = (uint32_t)tid * 4u;
-    } else if (SLOTS)
-        enc.init(col, lp, a.out + (stream / kSlotTile) * ((int64_t)kSlotTile * a.cap) + (stream % kSlotTile) * 4,
-                 kSlotTile * 4, a.cap);
-    else
-        enc.init(col, lp, a.out + id.row * a.o0 + id.ch * a.o1, 4, a.cap);
+        enc.init(col, lp);
+        enc.w.init(nullptr, 0, a.cap);
+        enc.w.init_tile(__builtin_amdgcn_make_buffer_rsrc((void *)(a.out + (int64_t)blockIdx.x * ((int64_t)kSlotTile * a.cap)), 0,
+                                                          kSlotTile * a.cap, kBufferWord3),
+                        (uint32_t)tid * 4u);
+    } else if (SLOTS) {
+        enc.init(col, lp);
+        enc.w.init(a.out + (stream / kSlotTile) * ((int64_t)kSlotTile * a.cap) + (stream % kSlotTile) * 4, kSlotTile * 4, a.cap);
+    } else {
+        enc.init(col, lp);
+        enc.w.init(a.out + id.row * a.o0 + id.ch * a.o1, 4, a.cap);
+    }
 
     // The row's alphabet (2C + 1 symbols for `bins` levels, encoder.py:44-52) may leave the
     // table's last symbol unused; then its special upper bound is never needed.  Uniform
@@ -379,7 +440,7 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
                         if (t + 6 < id.n) enc.template put_symbol<SENTINEL, false>((u >> 16) & 0xFFu);
                         if (t + 7 < id.n) enc.template put_symbol<SENTINEL, false>(u >> 24);
                     }
-                    enc.w.flush_word();
+                    enc.end_group();
                 }
             }
         } else {
@@ -397,7 +458,7 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
                 for (int j = 0; j < 8; j += 2) {
                     if (i0 + j < id.n) enc.template put_symbol<SENTINEL, true>(cur[j]);
                     if (i0 + j + 1 < id.n) enc.template put_symbol<SENTINEL, false>(cur[j + 1]);
-                    enc.w.flush_word();
+                    enc.end_group();
                 }
             }
         }

@@ -1,7 +1,8 @@
 """The HIP kernels do not run the reference's one-bit-at-a-time loops: they renormalise by a
-shift count taken from two count-leading-zero operations, splice pending bits in arithmetically,
-track the decoder's code value relative to the interval's low end, take the interval bounds from
-a high multiply and leave one bit of the decoder's `low` unmasked.  This module restates exactly
+shift count taken from two count-leading-zero operations, write the encoder's output as the
+interval's lower end with carries instead of counting pending bits, track the decoder's code
+value relative to the interval's low end, take the interval bounds from a high multiply and
+leave bit 31 of `low` as it falls.  This module restates exactly
 that arithmetic on Python integers (cachegen_amd/csrc/encoder.hpp: RangeEncoder::put_symbol,
 decoder.hpp: decode_symbol) and checks it, on the CPU, against the independent bit-serial coder
 of tests/pycoder.py: same bytes out of the encoder, same symbols out of the decoder, for tables
@@ -38,32 +39,78 @@ def shift_count(low, high):
     return n1, clz32(z)
 
 
-def model_encode(cdf, symbols):
-    bits = []                                              # emitted bits, as (value, count) pairs
-    low, span, pend = 0, 0, 0
-    for s in symbols:
+def model_encode(cdf, symbols, group=8):
+    """RangeEncoder: the interval's lower end is one long number, `low` (its last 32 bits, the
+    coder's window) below `out` (bits waiting to be written, at most 63 and a carry above them);
+    a symbol adds its offset and shifts the number left by the step count; complete words leave
+    once per `group` symbols through a held-back word that takes the carry, words of all ones
+    being counted until the word after them shows whether a carry comes."""
+    out, low, span, nout = 0, 0, 0, 0
+    cache, ones, words, started = 0, 0, [], [False]
+
+    def store(word):
+        if not started[0]:                                 # the empty held-back word of the start
+            started[0] = True
+            assert word == 0
+            return
+        assert 0 <= word <= M32
+        words.append(word)
+
+    def release(carry):
+        nonlocal ones
+        store(cache + carry)
+        for _ in range(ones):
+            store(0 if carry else M32)
+        ones = 0
+
+    def flush_word():
+        nonlocal out, nout, cache, ones
+        sh = nout - 32
+        word, carry = (out >> sh) & M32, out >> (sh + 32)
+        assert carry in (0, 1)
+        out &= (1 << sh) - 1
+        nout = sh
+        if ones == 0 and word != M32:
+            store(cache + carry)
+            cache = word
+        elif carry:
+            release(1)
+            cache = word
+        elif word == M32:
+            ones += 1
+        else:
+            release(0)
+            cache = word
+
+    def add_low(t):
+        nonlocal out, low
+        total = low + t
+        low, out = total & M32, out + (total >> 32)
+
+    def shift(n):
+        nonlocal out, low, nout
+        if nout + n + 1 > 64:
+            flush_word()
+        big = ((out << 32) | low) << n
+        low, out, nout = big & M32, big >> 32, nout + n
+        assert out < 1 << 64
+
+    for i, s in enumerate(symbols):
         t_lo, width = bound(cdf, s, span)
-        low = (low + t_lo) & M32
-        high = (low + width - 1) & M32
+        add_low(t_lo)
+        high = (low + width - 1) & M32                     # bit 31 of low may differ from the reference's
         n1, k = shift_count(low, high)
-        pe = pend if n1 > 0 else 0
-        m = n1 + pe
-        if n1 > 0:
-            top = low >> (32 - n1)                         # v_bfe_u32(low, 32 - n1, n1)
-            fill = ((1 << pe) - 1) << (n1 - 1)             # v_bfm_b32(pe, n1 - 1) when pe <= 31
-            bits.append((top + fill, m))
-        pend = pend - pe + k
-        low = (low << (n1 + k)) & 0x7FFFFFFF
+        shift(n1 + k)
         span = (width << (n1 + k)) & M32
-    pend += 1
-    first = 0 if low < 0x40000000 else 1
-    bits.append((first, 1))
-    bits.append((0 if first else (1 << pend) - 1, pend))
-    acc, nacc = 0, 0
-    for v, m in bits:
-        acc, nacc = (acc << m) | v, nacc + m
-    pad = -nacc % 8
-    return (acc << pad).to_bytes((nacc + pad) // 8, "big")
+        if i % group == group - 1 and nout >= 32:
+            flush_word()
+    add_low(0x40000000)
+    shift(2)
+    if nout >= 32:
+        flush_word()
+    release(out >> nout)
+    part = ((out & ((1 << nout) - 1)) << (32 - nout)) if nout else 0
+    return b"".join(w.to_bytes(4, "big") for w in words) + part.to_bytes(4, "big")[:(nout + 7) // 8]
 
 
 def model_decode(cdf, data, n):
@@ -142,3 +189,31 @@ def test_dyadic_table_hits_the_full_range_again():
     want, _ = pycoder.encode(cdf, syms)
     assert model_encode(cdf, syms) == want
     assert model_decode(cdf, want, len(syms)) == syms
+
+
+def test_carries_through_words_of_all_ones():
+    """Streams whose lower end runs 0111...1 over several words (the reference counts hundreds of
+    pending bits) and is then pushed over the edge, or not, by the symbols that follow."""
+    for width in (1, 2, 5):
+        cdf = [0, 65535 - width, 65535]
+        for n in (3, 10, 40):
+            for tail in ([], [0], [1, 0], [0, 0, 1]):
+                syms = [1] * n + tail
+                assert model_encode(cdf, syms) == pycoder.encode(cdf, syms)[0]
+    cdf = [0, 32767, 32768, 65535]
+    for n in range(1, 40):
+        for last in (0, 1, 2):
+            syms = [0] + [1] * n + [last, 2, 0, 1]
+            want = pycoder.encode(cdf, syms)[0]
+            assert model_encode(cdf, syms) == want
+            assert model_decode(cdf, want, len(syms)) == syms
+
+
+@pytest.mark.parametrize("group", [1, 2, 8])
+def test_word_schedule_does_not_change_the_stream(group):
+    rng = random.Random(group)
+    for _ in range(30):
+        nsym = rng.choice([3, 15, 31])
+        cdf = random_table(rng, nsym, rng.choice([1, 8]))
+        syms = [rng.randrange(nsym) for _ in range(rng.choice([5, 64, 300]))]
+        assert model_encode(cdf, syms, group) == pycoder.encode(cdf, syms)[0]

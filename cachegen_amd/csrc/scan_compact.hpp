@@ -37,6 +37,31 @@ __device__ __forceinline__ int64_t block_exclusive_scan(int64_t v, int64_t *lds,
     return incl - v;
 }
 
+// The same for a block of 256 threads and 32-bit values, with wavefront shuffles and one
+// exchange of the four wavefront totals through `lds` (at least 4 words).
+__device__ __forceinline__ int32_t block_exclusive_scan_256(int32_t v, int32_t *lds, int32_t &total)
+{
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    int32_t incl = v;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const int32_t up = __shfl_up(incl, o, 64);
+        if (lane >= o) incl += up;
+    }
+    if (lane == 63) lds[wave] = incl;
+    __syncthreads();
+    int32_t before = incl - v;
+    total = 0;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        const int32_t t = lds[w];
+        if (w < wave) before += t;
+        total += t;
+    }
+    __syncthreads();
+    return before;
+}
+
 __global__ __launch_bounds__(kScanThreads) void scan_tile_sums_kernel(
     const int32_t *__restrict__ lengths, int64_t n, int32_t clamp, int64_t *__restrict__ sums)
 {
@@ -187,12 +212,12 @@ __global__ __launch_bounds__(256) void compact_streams_kernel(
             mine = lengths[sbase + tid];
             mine = mine < 0 ? 0 : (mine > cap ? cap : mine);
         }
-        int64_t *lds = reinterpret_cast<int64_t *>(buf);       // kScanThreads values; buf is free until the copy
-        int64_t total64;
-        const int32_t before = (int32_t)block_exclusive_scan(mine, lds, total64);
         o0 = tile_base[blockIdx.x];
+        int32_t total32;
+        const int32_t before = block_exclusive_scan_256(mine, reinterpret_cast<int32_t *>(buf), total32);    // buf is free until the copy
+        const int64_t total64 = total32;                       // at most 256 streams of `cap` <= 256 bytes
         rel[tid] = before;
-        if (tid == 0) rel[kCompactStreams] = (int32_t)total64;
+        if (tid == 0) rel[kCompactStreams] = total32;
         if (tid < count) offsets[sbase + tid] = o0 + before;
         if (sbase + count == nstreams && tid == 0) offsets[nstreams] = o0 + total64;
         __syncthreads();

@@ -293,3 +293,60 @@ def test_streams_with_bogus_offsets_do_not_disturb_their_neighbours():
     got = out.reshape(L, 2, T, C).permute(1, 0, 3, 2).reshape(nstreams, T).cpu()
     want = clean.reshape(L, 2, T, C).permute(1, 0, 3, 2).reshape(nstreams, T).cpu()
     assert torch.equal(got[keep].view(torch.int16), want[keep].view(torch.int16))
+
+
+def _carry_cases():
+    """(table, symbols) pairs whose output runs 0111...1 over one or more whole words (hundreds
+    of pending bits in the reference's terms) and is then pushed over the edge by a carry, or
+    not, by the symbols that follow."""
+    cases = []
+    for width in (1, 2, 5):
+        cdf = [0, 1, 65535 - width, 65535]                  # the last symbol is tiny and at the very top
+        for n in (3, 10, 40):
+            for tail in ([], [1], [2, 1], [1, 1, 2], [0]):
+                cases.append((cdf, [2] * n + tail))
+    cdf = [0, 32767, 32768, 65535]                          # the middle symbol sits just below one half
+    for n in (1, 2, 5, 17, 31, 32, 33, 39):
+        for last in (0, 1, 2):
+            cases.append((cdf, [0] + [1] * n + [last, 2, 0, 1]))
+    cdf = [0, 32767, 32769, 65535]                          # the middle symbol straddles one half: every
+    for n in (1, 2, 3, 5, 8, 20):                           # repeat adds about fifteen undecided bits
+        for last in (0, 1, 2):
+            cases.append((cdf, [1] * n + [last, 0, 2]))
+    return cases
+
+
+@pytest.mark.gpu
+def test_carries_through_whole_words_of_ones_match_oracle(oracle):
+    """The encoder keeps the last complete word back until it knows whether a carry reaches it and
+    counts words of all ones behind it: streams that take those paths, through the reference's
+    entry point and byte for byte against the oracle's bit-serial pending count."""
+    from cachegen_amd import torchac_hip as tac
+    cases = _carry_cases()
+    nt = max(len(s) for _, s in cases)
+    nc = len(cases)
+    # every stream is padded with the wide symbol of its own table to the common length
+    sym = np.zeros((1, nt, nc), dtype=np.uint8)
+    cdf = np.zeros((1, nc, 4), dtype=np.uint16)
+    want = []
+    for c, (table, symbols) in enumerate(cases):
+        wide = max(range(3), key=lambda s: (table + [65536])[s + 1] - table[s])
+        padded = symbols + [wide] * (nt - len(symbols))
+        sym[0, :, c] = padded
+        cdf[0, c] = table
+        data, n = oracle.encode_stream(table, padded)
+        assert n <= 256
+        want.append(bytes(data))
+    assert any(b"\xff\xff\xff\xff" in w for w in want) and any(b"\x00\x00\x00\x00" in w for w in want)
+    out = torch.zeros((1, nc, 256), dtype=torch.uint8, device=DEV)
+    lengths = torch.zeros((1, nc), dtype=torch.int32, device=DEV)
+    tac.encode_fast_new(torch.from_numpy(cdf.view(np.int16)).to(DEV), torch.from_numpy(sym.view(np.int8)).to(DEV), out, lengths)
+    got_len = lengths.cpu().numpy()[0]
+    got = out.cpu().numpy()[0]
+    for c, w in enumerate(want):
+        assert got_len[c] == len(w), (c, cases[c])
+        assert bytes(got[c, :len(w)]) == w, (c, cases[c])
+    # and back
+    dec = torch.zeros((1, nt, nc), dtype=torch.uint8, device=DEV)
+    tac.decode_fast_new(torch.from_numpy(cdf.view(np.int16)).to(DEV), out, lengths, dec)
+    assert np.array_equal(dec.cpu().numpy(), sym)

@@ -321,7 +321,7 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
     const StreamId id = locate<BS>(a.sg);
     const int lp = a.lp;
     const int64_t ch0 = id.ch - tid;
-    uint16_t *col = tab + tid;
+    uint16_t *col = tab + table_column<BS>(tid);
     uint16_t *cdf_block = a.cdf + ((id.chunk * a.sg.rows + id.row) * a.sg.nc + ch0) * lp;
     const int nwords = (id.n + 3) >> 2;
     // PACKED: the sub-chunk's words ([word][channel]) are read through a buffer descriptor that
@@ -354,12 +354,13 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
 
     if (FUSE_CDF) {
         for (int i = 0; i < lp; ++i) col[i * TableStride<BS>::k16] = 0;
+        __syncthreads();                     // another lane, of another wavefront, shares this lane's words
         if (id.active) {
             const uint32_t smax = (uint32_t)(lp - 2);
             // two lanes share a 32-bit LDS word: each adds to its own half with one atomic that
             // returns nothing (a count is at most 256, so the low half never carries over)
-            uint32_t *const pair = reinterpret_cast<uint32_t *>(tab) + (tid >> 1);
-            const uint32_t one = (tid & 1) ? 0x10000u : 1u;
+            uint32_t *const pair = reinterpret_cast<uint32_t *>(tab) + (table_column<BS>(tid) >> 1);
+            const uint32_t one = (table_column<BS>(tid) & 1) ? 0x10000u : 1u;
             for (int h = 0; h * 32 < nwords; ++h) {
                 load_half(h);
                 // uniform; kept in a scalar register so that the loop test is scalar too
@@ -375,8 +376,9 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
                     }
                 }
             }
-            normalize_column16<BS>(col, lp, lp - 1, (uint32_t)id.n);
         }
+        __syncthreads();                     // the other lane's counts are all in
+        if (id.active) normalize_column16<BS>(col, lp, lp - 1, (uint32_t)id.n);
         __syncthreads();
         write_tables16<BS>(tab, cdf_block, lp, ch0, a.sg.nc);
     } else {

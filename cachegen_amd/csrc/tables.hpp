@@ -30,6 +30,16 @@ struct TableStride {
     static constexpr int k32 = BS + 1;      // 32-bit entries
 };
 
+// Column of lane c in a block's 16-bit tables: lanes c and c + BS/2 share a 32-bit word (low
+// and high half).  The two belong to different wavefronts (for blocks of 128 lanes or more), so
+// the lanes of one wavefront never add to the same word in one instruction when they count
+// symbols, and their look-ups spread over 64 words instead of 32.
+template <int BS>
+__device__ __forceinline__ int table_column(int c)
+{
+    return ((c & (BS / 2 - 1)) << 1) | (c / (BS / 2));
+}
+
 // Walks i = start, start + step, ... over tables stored one after the other ([channel][lp]) and
 // keeps (c, e) = (i / lp, i % lp) up to date with one divide at the start instead of one per step.
 struct TableWalk {
@@ -110,7 +120,7 @@ __device__ __forceinline__ void stage_tables16(uint16_t *tab, const uint16_t *cd
         for (int j = 0; j < kBatch; ++j) v[j] = i0 + j * BS < total ? cdf[i0 + j * BS] : (uint16_t)0;
 #pragma unroll
         for (int j = 0; j < kBatch; ++j) {
-            if (i0 + j * BS < total) tab[w.e * TableStride<BS>::k16 + w.c] = v[j];
+            if (i0 + j * BS < total) tab[w.e * TableStride<BS>::k16 + table_column<BS>(w.c)] = v[j];
             w.next(lp);
         }
     }
@@ -123,7 +133,7 @@ __device__ __forceinline__ void write_tables16(const uint16_t *tab, uint16_t *cd
     const int total = (int)nvalid * lp;
     TableWalk w(threadIdx.x, BS, lp);
     for (int i = threadIdx.x; i < total; i += BS, w.next(lp)) {
-        cdf[i] = tab[w.e * TableStride<BS>::k16 + w.c];
+        cdf[i] = tab[w.e * TableStride<BS>::k16 + table_column<BS>(w.c)];
     }
 }
 
@@ -185,9 +195,10 @@ __global__ __launch_bounds__(BS) void calculate_cdf_kernel(CdfArgs a)
     constexpr int kS16 = TableStride<BS>::k16, kS32 = TableStride<BS>::k32;
     uint32_t *col = smem + tid;
     uint16_t *tab16 = reinterpret_cast<uint16_t *>(smem);
+    const int tcol = table_column<BS>(tid);
     if (PACKED) {
-        for (int i = 0; i < lp; ++i) tab16[i * kS16 + tid] = 0;
-        __syncthreads();                     // a lane's neighbour shares its words
+        for (int i = 0; i < lp; ++i) tab16[i * kS16 + tcol] = 0;
+        __syncthreads();                     // another lane shares this lane's words
     } else {
         for (int i = 0; i < lp; ++i) col[i * kS32] = 0;
     }
@@ -213,8 +224,8 @@ __global__ __launch_bounds__(BS) void calculate_cdf_kernel(CdfArgs a)
                 if (v < mb) atomicAdd(col + (v + 1) * kS32, 1u);
             }
         } else {
-            uint32_t *const pair = smem + (tid >> 1);
-            const uint32_t one = (tid & 1) ? 0x10000u : 1u;
+            uint32_t *const pair = smem + (tcol >> 1);
+            const uint32_t one = (tcol & 1) ? 0x10000u : 1u;
             const int64_t sub0 = chunk * a.g.nsc;
             const int nsubs = (int)((t1 - t0 + kSub - 1) / kSub);
             for (int sidx = 0; sidx < nsubs; ++sidx) {
@@ -241,8 +252,8 @@ __global__ __launch_bounds__(BS) void calculate_cdf_kernel(CdfArgs a)
     const int64_t ch0 = (int64_t)ctile * BS;
     uint16_t *dst = a.cdf + ((chunk * a.rows + row) * a.nc + ch0) * lp;
     if (PACKED) {
-        __syncthreads();                     // the neighbour's atomics on the shared words are done
-        if (ch < a.nc) normalize_column16<BS>(tab16 + tid, lp, a.max_bins, (uint32_t)(t1 - t0));
+        __syncthreads();                     // the other lane's atomics on the shared words are done
+        if (ch < a.nc) normalize_column16<BS>(tab16 + tcol, lp, a.max_bins, (uint32_t)(t1 - t0));
         __syncthreads();
         write_tables16<BS>(tab16, dst, lp, ch0, a.nc);
     } else {

@@ -21,6 +21,7 @@
 #include <climits>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 
@@ -307,8 +308,11 @@ struct LevelOut {
 // symbols [2L, T, C]): calculate_cdf + encode_fast_new + collect_bytes for every chunk
 // (encoder.py:265-292, 209-222).
 // The level's status word has been set to zero by an earlier launch of the same call.
+// maxima, max_dt: the row maxima (packed symbols only); nibbles: the quantizer packed the rows
+// of at most 15 symbols four bits a symbol (see packs_nibbles).
 int code_and_compact(const LevelOut &o, const uint32_t *sym4, const uint8_t *sym_bytes, const EncodeWorkspace &w,
-                     int64_t L, int64_t T, int64_t C, int64_t chunk_tokens, hipStream_t s)
+                     int64_t L, int64_t T, int64_t C, int64_t chunk_tokens, hipStream_t s,
+                     const void *maxima = nullptr, int max_dt = 0, bool nibbles = false)
 {
     const int64_t rows = 2 * L;
     const int lp = o.max_bins + 1;
@@ -339,6 +343,9 @@ int code_and_compact(const LevelOut &o, const uint32_t *sym4, const uint8_t *sym
     if (sym4) {
         // four tokens per word, read by one lane per channel
         a.sym4 = sym4;
+        a.nibbles = nibbles ? 1 : 0;
+        a.maxima = static_cast<const uint16_t *>(maxima);
+        a.max_dt = max_dt;
         if (chunk_tokens <= kSub) {
             // one sub-chunk per chunk: the encoder builds the tables itself
             if (fused_scan) encode_streams_kernel<kSlotTile, true, true, true, true, true><<<grid, blk, shmem, s>>>(a);
@@ -372,6 +379,11 @@ int code_and_compact(const LevelOut &o, const uint32_t *sym4, const uint8_t *sym
             w.scratch, kStreamCap, o.offsets, nullptr, nullptr, w.nstreams, o.payload, o.payload_cap, skew, o.status);
     }
     return check_launch("compact");
+}
+
+bool packs_nibbles(int64_t chunk_tokens, int delta_group)
+{
+    return chunk_tokens <= kSub && delta_group == 0 && !getenv("CG_ENCODE_BYTES");
 }
 
 int check_kv_geometry(const char *what, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D, int64_t chunk_tokens)
@@ -410,9 +422,13 @@ int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int
         return fail(CG_ERR_ARG, "encode_kv: delta groups need head sizes and strides that are multiples of 8 and a 16-byte aligned tensor");
     if (packed) {
         uint32_t *sym4 = reinterpret_cast<uint32_t *>(w.symbols);
+        // one sub-chunk per chunk (the coder reads the symbols itself, twice): rows of at most 15
+        // symbols travel four bits a symbol
+        const bool nibbles = packs_nibbles(chunk_tokens, delta_group);
         if (int rc = launch_quantize_pack(kv, kv_dt, L, T, H, D, sl, skv, st, sh, key_bins, value_bins, sym4,
-                                          maxima, w.nsub, chunk_tokens, delta_group, s, status)) return rc;
-        return code_and_compact(o, sym4, nullptr, w, L, T, C, chunk_tokens, s);
+                                          maxima, w.nsub, chunk_tokens, delta_group, s, status, 0, nullptr, nullptr, 0,
+                                          nibbles)) return rc;
+        return code_and_compact(o, sym4, nullptr, w, L, T, C, chunk_tokens, s, maxima, kv_dt, nibbles);
     }
     clear_status_kernel<<<1, 1, 0, s>>>(status);
     if (int rc = launch_quantize(kv, kv_dt, L, T, H, D, sl, skv, st, sh, key_bins, value_bins, w.symbols, maxima, s)) return rc;
@@ -457,7 +473,7 @@ int cg_encode_kv_levels(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t
                             payload[v], payload_cap[v], status + v};
         uint8_t *symbols = w.symbols + (size_t)v * w.symbols_bytes;
         if (packed) {
-            if (int rc = code_and_compact(o, reinterpret_cast<uint32_t *>(symbols), nullptr, w, L, T, C, chunk_tokens, s)) return rc;
+            if (int rc = code_and_compact(o, reinterpret_cast<uint32_t *>(symbols), nullptr, w, L, T, C, chunk_tokens, s, maxima, kv_dt)) return rc;
         } else {
             // shapes the vector loads cannot take: one plain quantization pass per level
             clear_status_kernel<<<1, 1, 0, s>>>(status + v);

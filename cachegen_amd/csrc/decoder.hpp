@@ -407,7 +407,8 @@ __global__ __launch_bounds__(BS) void decode_streams_kernel(DecodeArgs a)
         const uint16_t *mx = a.maxima + id.row * a.sg.g.T + id.t0;
         for (int i = tid; i < id.n; i += BS) {
             const float m = a.max_dt == CG_DT_BF16 ? load16f<CG_DT_BF16>(mx[i]) : load16f<CG_DT_F16>(mx[i]);
-            special |= (__float_as_uint(m) & 0x7FFFFFFFu) >= 0x7F800000u;
+            // also rows whose scale overflowed in the quantizer: they hold the table's last symbol
+            special |= (__float_as_uint(m) & 0x7FFFFFFFu) >= 0x7F800000u || scale_overflows(cq, m);
             rowmax[i] = m;
         }
     }

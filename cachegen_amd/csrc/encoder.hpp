@@ -242,10 +242,12 @@ struct RangeEncoder {
     // SENTINEL: symbol smax may occur, whose upper bound is 2^16 and not the table's last
     // entry (enc_new.cu:270)
     // FIRST: the symbol directly follows a flush (the first of a group)
-    template <bool SENTINEL, bool FIRST>
+    // CLAMP: the symbol may lie outside the table (it is kept inside; symbols that are known to
+    // be table symbols skip the compare)
+    template <bool SENTINEL, bool FIRST, bool CLAMP = true>
     __device__ __forceinline__ void put_symbol(uint32_t s)
     {
-        s = s < smax ? s : smax;                        // keep table reads inside the table
+        if (CLAMP) s = s < smax ? s : smax;             // keep table reads inside the table
         constexpr int kRow = 2 * TableStride<BS>::k16;
         lds_entries_high<kRow>(col + s * kRow, bound_lo, bound_hi);
         // the upper bound of symbol smax is 2^16 and not the table's last entry; shifted left
@@ -292,6 +294,9 @@ struct EncodeArgs {
     const uint8_t *sym;     // byte symbols: sym[row*s0 + token*s1 + channel*s2]
     int64_t s0, s1, s2;
     const uint32_t *sym4;   // or packed symbols
+    int32_t nibbles;        // rows of at most 15 symbols are packed four bits a symbol (quantize_pack_kernel)
+    const uint16_t *maxima; // the row maxima [2L, T] and their type, to know the rows that saturate (or null)
+    int32_t max_dt;
     int64_t nsub;
     uint8_t *out;           // out[row*o0 + channel*o1 + byte], or the scratch tiles (SLOTS)
     int64_t o0, o1;
@@ -309,6 +314,26 @@ template <bool B>
 struct BoolTag {
     static constexpr bool value = B;
 };
+
+// How a packed word holds its four symbols: kBytes, a byte each (any value; kept inside the
+// table where it is used); kNibbles, four bits each, every one a table symbol; kNibblesEscaped,
+// four bits each where 15 stands for a saturated byte, i.e. the table's last symbol.
+enum { kBytes = 0, kNibbles = 1, kNibblesEscaped = 2 };
+
+template <bool SENTINEL_, int MODE_>
+struct CodeTag {
+    static constexpr bool SENTINEL = SENTINEL_;
+    static constexpr int MODE = MODE_;
+};
+
+template <int MODE>
+__device__ __forceinline__ uint32_t packed_symbol(uint32_t v, int j, uint32_t smax)
+{
+    if (MODE == kBytes) return (v >> (8 * j)) & 0xFFu;
+    uint32_t s = __builtin_amdgcn_ubfe(v, (uint32_t)(4 * j), 4u);
+    if (MODE == kNibblesEscaped) s = s == 15u ? smax : s;
+    return s;
+}
 
 // PACKED: symbols come from sym4.  FUSE_CDF (PACKED only, one sub-chunk per chunk): the
 // block first builds its own tables from the same words and writes them out.
@@ -339,6 +364,34 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
                                                          (int)((uint32_t)nwords * row_bytes), kBufferWord3);
         if (id.active) symbols_voff = (uint32_t)id.ch * 4u;
     }
+    // The row's alphabet (2C + 1 symbols for `bins` levels, encoder.py:44-52): it may leave the
+    // table's last symbol unused (then its special upper bound is never needed), and with at
+    // most 15 symbols the quantizer may have packed it four bits a symbol, two channels to a
+    // word.  A token row whose scale overflowed (a maximum so small that MAX / max is infinite)
+    // saturates its bytes to 255, which the reference's coder reads as the table's last symbol:
+    // such bytes arrive as the value 15.  All uniform over the block.
+    bool sentinel = true;
+    int mode = kBytes;
+    uint32_t half_shift = 0;
+    if (PACKED && a.key_bins) {
+        const int64_t kvi = id.row / a.L, l = id.row - kvi * a.L;
+        const float cq = floorf((kvi ? a.value_bins : a.key_bins)[l] * 0.5f) - 1.0f;
+        sentinel = !(cq >= 0.0f && 2.0f * cq + 1.0f <= (float)(lp - 2));
+        if (a.maxima) {
+            int saturates = 0;
+            if (tid < id.n) {
+                const uint32_t bits = a.maxima[id.row * a.sg.g.T + id.t0 + tid];
+                const float m = a.max_dt == CG_DT_BF16 ? load16f<CG_DT_BF16>(bits) : load16f<CG_DT_F16>(bits);
+                saturates = scale_overflows(cq, m);
+            }
+            if (__syncthreads_or(saturates)) sentinel = true;       // the last symbol does occur
+        }
+        if (a.nibbles && narrow_alphabet(cq)) {
+            mode = sentinel ? kNibblesEscaped : kNibbles;
+            if (id.active) symbols_voff = (uint32_t)(id.ch >> 1) * 4u;
+            half_shift = (uint32_t)(id.ch & 1) * 16u;
+        }
+    }
 
     // Half a sub-chunk (32 words = 128 symbols) at a time is loaded into registers and indexed
     // by the (uniform) loop counter, so the coding loop has no loads to wait for and its stores
@@ -361,21 +414,27 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
             // returns nothing (a count is at most 256, so the low half never carries over)
             uint32_t *const pair = reinterpret_cast<uint32_t *>(tab) + (table_column<BS>(tid) >> 1);
             const uint32_t one = (table_column<BS>(tid) & 1) ? 0x10000u : 1u;
-            for (int h = 0; h * 32 < nwords; ++h) {
-                load_half(h);
-                // uniform; kept in a scalar register so that the loop test is scalar too
-                const int wn = __builtin_amdgcn_readfirstlane(nwords - h * 32 < 32 ? nwords - h * 32 : 32);
+            auto count = [&](auto tag) {
+                constexpr int MODE = decltype(tag)::MODE;
+                for (int h = 0; h * 32 < nwords; ++h) {
+                    load_half(h);
+                    // uniform; kept in a scalar register so that the loop test is scalar too
+                    const int wn = __builtin_amdgcn_readfirstlane(nwords - h * 32 < 32 ? nwords - h * 32 : 32);
 #pragma unroll 1
-                for (int w = 0; w < wn; ++w) {
-                    const uint32_t v = words[w];
+                    for (int w = 0; w < wn; ++w) {
+                        const uint32_t v = MODE == kBytes ? words[w] : words[w] >> half_shift;
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        uint32_t s = (v >> (8 * j)) & 0xFFu;
-                        s = s < smax ? s : smax;
-                        if ((h * 32 + w) * 4 + j < id.n) atomicAdd(pair + (s + 1) * (TableStride<BS>::k16 / 2), one);
+                        for (int j = 0; j < 4; ++j) {
+                            uint32_t s = packed_symbol<MODE>(v, j, smax);
+                            if (MODE == kBytes) s = s < smax ? s : smax;
+                            if ((h * 32 + w) * 4 + j < id.n) atomicAdd(pair + (s + 1) * (TableStride<BS>::k16 / 2), one);
+                        }
                     }
                 }
-            }
+            };
+            if (mode == kNibbles) count(CodeTag<false, kNibbles>());
+            else if (mode == kNibblesEscaped) count(CodeTag<false, kNibblesEscaped>());
+            else count(CodeTag<false, kBytes>());
         }
         __syncthreads();                     // the other lane's counts are all in
         if (id.active) normalize_column16<BS>(col, lp, lp - 1, (uint32_t)id.n);
@@ -408,18 +467,11 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
         enc.w.init(a.out + id.row * a.o0 + id.ch * a.o1, 4, a.cap);
     }
 
-    // The row's alphabet (2C + 1 symbols for `bins` levels, encoder.py:44-52) may leave the
-    // table's last symbol unused; then its special upper bound is never needed.  Uniform
-    // over the block.
-    bool sentinel = true;
-    if (PACKED && a.key_bins) {
-        const int64_t kvi = id.row / a.L, l = id.row - kvi * a.L;
-        const float cq = floorf((kvi ? a.value_bins : a.key_bins)[l] * 0.5f) - 1.0f;
-        sentinel = !(cq >= 0.0f && 2.0f * cq + 1.0f <= (float)(lp - 2));
-    }
-
     auto code = [&](auto tag) {
-        constexpr bool SENTINEL = decltype(tag)::value;
+        constexpr bool SENTINEL = decltype(tag)::SENTINEL;
+        constexpr int MODE = decltype(tag)::MODE;
+        constexpr bool CLAMP = MODE == kBytes;
+        const uint32_t smax = (uint32_t)(lp - 2);
         if (PACKED) {
             for (int h = 0; h * 32 < nwords; ++h) {
                 load_half(h);
@@ -429,18 +481,19 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
                 // except in a sub-chunk's last, partial run of words)
 #pragma unroll 1
                 for (int w = 0; w < wn; w += 2) {
-                    const uint32_t v = words[w];
+                    const uint32_t v = MODE == kBytes ? words[w] : words[w] >> half_shift;
                     const int t = (h * 32 + w) * 4;            // first token of the word
-                    if (t + 0 < id.n) enc.template put_symbol<SENTINEL, true>(v & 0xFFu);
-                    if (t + 1 < id.n) enc.template put_symbol<SENTINEL, false>((v >> 8) & 0xFFu);
-                    if (t + 2 < id.n) enc.template put_symbol<SENTINEL, false>((v >> 16) & 0xFFu);
-                    if (t + 3 < id.n) enc.template put_symbol<SENTINEL, false>(v >> 24);
+                    if (t + 0 < id.n) enc.template put_symbol<SENTINEL, true, CLAMP>(packed_symbol<MODE>(v, 0, smax));
+                    if (t + 1 < id.n) enc.template put_symbol<SENTINEL, false, CLAMP>(packed_symbol<MODE>(v, 1, smax));
+                    if (t + 2 < id.n) enc.template put_symbol<SENTINEL, false, CLAMP>(packed_symbol<MODE>(v, 2, smax));
+                    if (t + 3 < id.n) enc.template put_symbol<SENTINEL, false, CLAMP>(packed_symbol<MODE>(v, 3, smax));
                     if (t + 4 < id.n) {
-                        const uint32_t u = words[w + 1];       // w + 1 <= 31: wn <= 32
-                        enc.template put_symbol<SENTINEL, false>(u & 0xFFu);
-                        if (t + 5 < id.n) enc.template put_symbol<SENTINEL, false>((u >> 8) & 0xFFu);
-                        if (t + 6 < id.n) enc.template put_symbol<SENTINEL, false>((u >> 16) & 0xFFu);
-                        if (t + 7 < id.n) enc.template put_symbol<SENTINEL, false>(u >> 24);
+                        // w + 1 <= 31: wn <= 32
+                        const uint32_t u = MODE == kBytes ? words[w + 1] : words[w + 1] >> half_shift;
+                        enc.template put_symbol<SENTINEL, false, CLAMP>(packed_symbol<MODE>(u, 0, smax));
+                        if (t + 5 < id.n) enc.template put_symbol<SENTINEL, false, CLAMP>(packed_symbol<MODE>(u, 1, smax));
+                        if (t + 6 < id.n) enc.template put_symbol<SENTINEL, false, CLAMP>(packed_symbol<MODE>(u, 2, smax));
+                        if (t + 7 < id.n) enc.template put_symbol<SENTINEL, false, CLAMP>(packed_symbol<MODE>(u, 3, smax));
                     }
                     enc.end_group();
                 }
@@ -465,8 +518,10 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
             }
         }
     };
-    if (PACKED && !sentinel) code(BoolTag<false>());
-    else code(BoolTag<true>());
+    if (PACKED && mode == kNibbles) code(CodeTag<false, kNibbles>());
+    else if (PACKED && mode == kNibblesEscaped) code(CodeTag<true, kNibblesEscaped>());
+    else if (PACKED && !sentinel) code(CodeTag<false, kBytes>());
+    else code(CodeTag<true, kBytes>());
     const int len = enc.finish();
     a.lengths[stream] = len;
     if (len > a.cap && a.status) atomicOr(a.status, 1);

@@ -175,7 +175,7 @@ int launch_quantize_pack(const void *kv, int kv_dt, int64_t L, int64_t T, int64_
                          const float *value_bins, uint32_t *sym4, void *maxima, int64_t nsub,
                          int64_t S, int delta_group, hipStream_t stream, int32_t *status, int nlevels = 0,
                          const float *const *key_bins_lv = nullptr, const float *const *value_bins_lv = nullptr,
-                         int64_t level_words = 0)
+                         int64_t level_words = 0, bool nibbles = false)
 {
     PackedQuantArgs a;
     memset(&a, 0, sizeof(a));
@@ -188,6 +188,7 @@ int launch_quantize_pack(const void *kv, int kv_dt, int64_t L, int64_t T, int64_
         a.value_bins_lv[v] = value_bins_lv[v];
     }
     a.level_words = level_words;
+    a.nibbles = nibbles ? 1 : 0;
     a.kv = static_cast<const uint16_t *>(kv);
     a.L = L;
     a.sl = sl;

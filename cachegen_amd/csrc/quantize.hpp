@@ -171,6 +171,7 @@ struct PackedQuantArgs {
     uint16_t *maxima;       // [2L, T]
     int32_t nunits;         // C / 8
     int64_t nsub;
+    int32_t nibbles;        // rows of at most 15 symbols are written four bits a symbol (see quantize_pack_kernel)
     int32_t delta_group;    // > 0: tokens of a sub-chunk in groups of this many, see below
     TokenGeom g;
 };
@@ -184,6 +185,21 @@ struct PackedQuantArgs {
 __device__ __forceinline__ void clear_statuses(const PackedQuantArgs &a)
 {
     if (blockIdx.x == 0 && threadIdx.x < a.nstatus) *a.status[threadIdx.x] = 0;
+}
+
+// A row quantized to `maxq` levels either side of zero has the symbols 0 .. 2 maxq: at most
+// fifteen of them fit four bits with the value 15 to spare.  Where the caller asks for it
+// (a.nibbles) such rows are stored four bits a symbol, word w of channel pair p (channels 2p and
+// 2p + 1) of a sub-chunk at sym4[((row * nsub + sub) * 64 + w) * C + p]: half of the bytes.
+__device__ __forceinline__ bool narrow_alphabet(float maxq) { return maxq >= 0.0f && maxq <= 7.0f; }
+
+// A token row whose maximum is so small that the scale maxq / max is infinite (bfloat16 maxima
+// below about 2^-125): every non-zero value of the row saturates, to the byte 255, which the
+// coder keeps inside the table as the table's last symbol.  Rows of zeros do not count (0 * inf
+// is a NaN, symbol 0).
+__device__ __forceinline__ bool scale_overflows(float maxq, float row_max)
+{
+    return row_max != 0.0f && (__float_as_uint(__fdiv_rn(maxq, row_max)) & 0x7FFFFFFFu) == 0x7F800000u;
 }
 
 template <int DT, bool HEADS_CONTIGUOUS, int NU, bool MULTI = false>
@@ -241,6 +257,7 @@ __global__ __launch_bounds__(256) void quantize_pack_kernel(PackedQuantArgs a)
     for (int lv = 0; lv < nlevels; ++lv, out += a.level_words) {
         const float bins = MULTI ? (kvi ? a.value_bins_lv[lv] : a.key_bins_lv[lv])[l] : (kvi ? a.value_bins : a.key_bins)[l];
         const float maxq = floorf(bins * 0.5f) - 1.0f;
+        const bool narrow = a.nibbles && narrow_alphabet(maxq);
         float factor[4];
         // rows past the end of the sub-chunk are all zero: 0 * inf = NaN -> symbol byte 0
 #pragma unroll
@@ -267,9 +284,24 @@ __global__ __launch_bounds__(256) void quantize_pack_kernel(PackedQuantArgs a)
                     }
                     words[k] = w;
                 }
-                uint4 *dst = reinterpret_cast<uint4 *>(out + (int64_t)u * 8);
-                dst[0] = make_uint4(words[0], words[1], words[2], words[3]);
-                dst[1] = make_uint4(words[4], words[5], words[6], words[7]);
+                if (!MULTI && narrow) {
+                    // four bits a symbol: channels 2k and 2k + 1 share word k of the unit, the even
+                    // channel's four tokens in its lower half.  A saturated byte (255) becomes 15,
+                    // which no symbol of such a row is: the coder gives it its meaning back.
+                    uint32_t half[4];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        uint32_t e = words[2 * k] & 0x0F0F0F0Fu, o = words[2 * k + 1] & 0x0F0F0F0Fu;
+                        e |= e >> 4;                                    // bytes 0 and 2 hold two symbols each
+                        o |= o >> 4;
+                        half[k] = __builtin_amdgcn_perm(o, e, 0x06040200u);          // e.b0, e.b2, o.b0, o.b2
+                    }
+                    *reinterpret_cast<uint4 *>(out + (int64_t)u * 4) = make_uint4(half[0], half[1], half[2], half[3]);
+                } else {
+                    uint4 *dst = reinterpret_cast<uint4 *>(out + (int64_t)u * 8);
+                    dst[0] = make_uint4(words[0], words[1], words[2], words[3]);
+                    dst[1] = make_uint4(words[4], words[5], words[6], words[7]);
+                }
             }
         }
     }

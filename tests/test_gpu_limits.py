@@ -350,3 +350,50 @@ def test_carries_through_whole_words_of_ones_match_oracle(oracle):
     dec = torch.zeros((1, nt, nc), dtype=torch.uint8, device=DEV)
     tac.decode_fast_new(torch.from_numpy(cdf.view(np.int16)).to(DEV), out, lengths, dec)
     assert np.array_equal(dec.cpu().numpy(), sym)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_four_bit_symbol_words_give_the_same_streams_as_byte_words(dtype):
+    """Rows of at most 15 symbols cross from the quantizer to the coder four bits a symbol.  The
+    other form (a byte a symbol, CG_ENCODE_BYTES=1) must give the same tables, streams and maxima,
+    also for token rows whose scale overflows (bfloat16 maxima below 2^-125: MAX / max is
+    infinite, every non-zero value saturates to the table's last symbol) and rows of zeros."""
+    import os
+    codec, _ = _mods()
+    torch.manual_seed(11)
+    L, T, H, D = 3, 300, 4, 128
+    kv = torch.randn((L, 2, T, H, D), dtype=torch.float32)
+    kv[1, 0, 7] = 0.0                                       # a row of zeros
+    if dtype == torch.bfloat16:
+        kv[2, 1, 40:44] *= 1e-39                            # denormal maxima: the scale overflows
+        kv[0, 0, 299] *= 3e-39
+        kv[1, 1, 100] *= 1e-39
+    kv = kv.to(dtype).to(DEV)
+    kb = torch.tensor([32.0, 16.0, 12.0])
+    vb = torch.tensor([16.0, 8.0, 16.0])
+    assert "CG_ENCODE_BYTES" not in os.environ
+    got = codec.encode_kv(kv, kb, vb, chunk_tokens=256)
+    got.check()
+    os.environ["CG_ENCODE_BYTES"] = "1"
+    try:
+        ref = codec.encode_kv(kv, kb, vb, chunk_tokens=256)
+        ref.check()
+    finally:
+        del os.environ["CG_ENCODE_BYTES"]
+    n = ref.total_bytes()
+    assert got.total_bytes() == n
+    assert torch.equal(got.cdf, ref.cdf) and torch.equal(got.lengths, ref.lengths) and torch.equal(got.offsets, ref.offsets)
+    assert torch.equal(got.payload[:n], ref.payload[:n]) and torch.equal(got.maxima, ref.maxima)
+    if dtype == torch.bfloat16:
+        # the saturated rows really use the last table symbol (value layer 2 has 16 levels: symbol 31 of 33 entries)
+        last = ref.cdf[0, 3 + 2].to(torch.int32) & 0xFFFF   # row = L + layer 2
+        assert int((last[:, 32] - last[:, 31]).max()) > 1
+    # the decoder gives the coder's symbols back: every value within half a step of its row's scale
+    out = codec.decode_encoded(got, kb, vb, out_dtype=dtype).float().cpu()
+    src = kv.float().cpu()
+    mx = src.abs().amax(dim=(-1, -2), keepdim=True)
+    step = mx / (torch.floor(torch.cat([kb, vb]).view(2, L).t().reshape(L, 2, 1, 1, 1) / 2) - 1)
+    ok = (out - src).abs() <= 0.6 * step + 1e-30             # half a step and the 16-bit rounding of the output
+    sane = mx > 1e-30                                       # rows whose scale did not overflow
+    assert bool((ok | ~sane.expand_as(ok)).all())

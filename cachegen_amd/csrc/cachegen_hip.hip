@@ -351,7 +351,8 @@ int code_and_compact(const LevelOut &o, const uint32_t *sym4, const uint8_t *sym
             if (fused_scan) encode_streams_kernel<kSlotTile, true, true, true, true, true><<<grid, blk, shmem, s>>>(a);
             else CG_DISPATCH_BS(block, (encode_streams_kernel<BS, true, true, true, true><<<grid, blk, shmem, s>>>(a)));
         } else {
-            if (int rc = launch_cdf(nullptr, sym4, w.nsub, rows, T, C, 0, 0, 0, o.max_bins, chunk_tokens, tables, s)) return rc;
+            if (int rc = launch_cdf(nullptr, sym4, w.nsub, rows, T, C, 0, 0, 0, o.max_bins, chunk_tokens, tables, s,
+                                    nibbles ? o.key_bins : nullptr, nibbles ? o.value_bins : nullptr)) return rc;
             if (fused_scan) encode_streams_kernel<kSlotTile, true, true, false, true, true><<<grid, blk, shmem, s>>>(a);
             else CG_DISPATCH_BS(block, (encode_streams_kernel<BS, true, true, false, true><<<grid, blk, shmem, s>>>(a)));
         }
@@ -381,9 +382,9 @@ int code_and_compact(const LevelOut &o, const uint32_t *sym4, const uint8_t *sym
     return check_launch("compact");
 }
 
-bool packs_nibbles(int64_t chunk_tokens, int delta_group)
+bool packs_nibbles(int delta_group)
 {
-    return chunk_tokens <= kSub && delta_group == 0 && !getenv("CG_ENCODE_BYTES");
+    return delta_group == 0 && !getenv("CG_ENCODE_BYTES");
 }
 
 int check_kv_geometry(const char *what, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D, int64_t chunk_tokens)
@@ -422,9 +423,8 @@ int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int
         return fail(CG_ERR_ARG, "encode_kv: delta groups need head sizes and strides that are multiples of 8 and a 16-byte aligned tensor");
     if (packed) {
         uint32_t *sym4 = reinterpret_cast<uint32_t *>(w.symbols);
-        // one sub-chunk per chunk (the coder reads the symbols itself, twice): rows of at most 15
-        // symbols travel four bits a symbol
-        const bool nibbles = packs_nibbles(chunk_tokens, delta_group);
+        // rows of at most 15 symbols travel four bits a symbol
+        const bool nibbles = packs_nibbles(delta_group);
         if (int rc = launch_quantize_pack(kv, kv_dt, L, T, H, D, sl, skv, st, sh, key_bins, value_bins, sym4,
                                           maxima, w.nsub, chunk_tokens, delta_group, s, status, 0, nullptr, nullptr, 0,
                                           nibbles)) return rc;

@@ -46,9 +46,11 @@ int make_grid(int64_t rows, int64_t nc, int64_t T, int64_t S, int64_t nsub, int 
         else { constexpr int BS = 64; __VA_ARGS__; }    \
     } while (0)
 
+// key_bins, value_bins (packed symbols only, may be null): the rows of at most 15 symbols hold
+// four bits a symbol.
 int launch_cdf(const uint8_t *sym, const uint32_t *sym4, int64_t nsub, int64_t rows, int64_t T,
                int64_t nc, int64_t s0, int64_t s1, int64_t s2, int max_bins, int64_t S,
-               uint16_t *cdf, hipStream_t stream)
+               uint16_t *cdf, hipStream_t stream, const float *key_bins = nullptr, const float *value_bins = nullptr)
 {
     int block = pick_block(nc, max_bins + 1);
     while (!sym4 && block > 64 && (size_t)(max_bins + 1) * (block + 1) * sizeof(uint32_t) > 64 * 1024) block /= 2;
@@ -59,6 +61,10 @@ int launch_cdf(const uint8_t *sym, const uint32_t *sym4, int64_t nsub, int64_t r
     a.s2 = s2;
     a.sym4 = sym4;
     a.nsub = nsub;
+    a.nibbles = (sym4 && key_bins && value_bins) ? 1 : 0;
+    a.key_bins = key_bins;
+    a.value_bins = value_bins;
+    a.L = rows / 2;
     a.cdf = cdf;
     a.rows = rows;
     a.nc = nc;

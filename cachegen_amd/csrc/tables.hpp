@@ -171,6 +171,11 @@ struct CdfArgs {
     int64_t s0, s1, s2;
     const uint32_t *sym4;   // or packed symbols (see above)
     int64_t nsub;
+    // packed symbols: rows of at most 15 symbols hold four bits a symbol, two channels to a word
+    // (quantize_pack_kernel); the levels of the rows
+    int32_t nibbles;
+    const float *key_bins, *value_bins;
+    int64_t L;
     uint16_t *cdf;          // [chunk][row][channel][lp]
     int64_t rows, nc;
     int32_t ctiles;
@@ -227,22 +232,39 @@ __global__ __launch_bounds__(BS) void calculate_cdf_kernel(CdfArgs a)
             uint32_t *const pair = smem + (tcol >> 1);
             const uint32_t one = (tcol & 1) ? 0x10000u : 1u;
             const int64_t sub0 = chunk * a.g.nsc;
+            bool narrow = false;                     // uniform over the block
+            if (a.nibbles) {
+                const int64_t kvi = row / a.L, l = row - kvi * a.L;
+                narrow = narrow_alphabet(floorf((kvi ? a.value_bins : a.key_bins)[l] * 0.5f) - 1.0f);
+            }
+            const int64_t column = narrow ? (ch >> 1) : ch;
+            const uint32_t half_shift = narrow ? (uint32_t)(ch & 1) * 16u : 0u;
             const int nsubs = (int)((t1 - t0 + kSub - 1) / kSub);
             for (int sidx = 0; sidx < nsubs; ++sidx) {
                 const int64_t left = (t1 - t0) - (int64_t)sidx * kSub;
                 const int n = left < kSub ? (int)left : kSub;
-                const uint32_t *wp = a.sym4 + ((row * a.nsub + sub0 + sidx) * kWordsPerSub) * a.nc + ch;
+                const uint32_t *wp = a.sym4 + ((row * a.nsub + sub0 + sidx) * kWordsPerSub) * a.nc + column;
                 const int nwords = (n + 3) >> 2;
                 constexpr int kBatch = 16;          // words in flight per lane
                 for (int w0 = 0; w0 < nwords; w0 += kBatch) {
                     uint32_t v[kBatch];
 #pragma unroll
                     for (int j = 0; j < kBatch; ++j) v[j] = (w0 + j < nwords) ? wp[(int64_t)(w0 + j) * a.nc] : 0u;
+                    if (narrow) {
+                        // the value 15 stands for a saturated byte: the table's last symbol
 #pragma unroll
-                    for (int j = 0; j < 4 * kBatch; ++j) {
-                        uint32_t s = (v[j >> 2] >> (8 * (j & 3))) & 0xFFu;
-                        s = s < mb - 1u ? s : mb - 1u;
-                        if (w0 * 4 + j < n) atomicAdd(pair + (s + 1) * (kS16 / 2), one);
+                        for (int j = 0; j < 4 * kBatch; ++j) {
+                            uint32_t s = __builtin_amdgcn_ubfe(v[j >> 2] >> half_shift, (uint32_t)(4 * (j & 3)), 4u);
+                            s = s == 15u ? mb - 1u : s;
+                            if (w0 * 4 + j < n) atomicAdd(pair + (s + 1) * (kS16 / 2), one);
+                        }
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 4 * kBatch; ++j) {
+                            uint32_t s = (v[j >> 2] >> (8 * (j & 3))) & 0xFFu;
+                            s = s < mb - 1u ? s : mb - 1u;
+                            if (w0 * 4 + j < n) atomicAdd(pair + (s + 1) * (kS16 / 2), one);
+                        }
                     }
                 }
             }

@@ -353,8 +353,9 @@ def test_carries_through_whole_words_of_ones_match_oracle(oracle):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("chunk", [256, 300])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-def test_four_bit_symbol_words_give_the_same_streams_as_byte_words(dtype):
+def test_four_bit_symbol_words_give_the_same_streams_as_byte_words(dtype, chunk):
     """Rows of at most 15 symbols cross from the quantizer to the coder four bits a symbol.  The
     other form (a byte a symbol, CG_ENCODE_BYTES=1) must give the same tables, streams and maxima,
     also for token rows whose scale overflows (bfloat16 maxima below 2^-125: MAX / max is
@@ -373,11 +374,11 @@ def test_four_bit_symbol_words_give_the_same_streams_as_byte_words(dtype):
     kb = torch.tensor([32.0, 16.0, 12.0])
     vb = torch.tensor([16.0, 8.0, 16.0])
     assert "CG_ENCODE_BYTES" not in os.environ
-    got = codec.encode_kv(kv, kb, vb, chunk_tokens=256)
+    got = codec.encode_kv(kv, kb, vb, chunk_tokens=chunk)
     got.check()
     os.environ["CG_ENCODE_BYTES"] = "1"
     try:
-        ref = codec.encode_kv(kv, kb, vb, chunk_tokens=256)
+        ref = codec.encode_kv(kv, kb, vb, chunk_tokens=chunk)
         ref.check()
     finally:
         del os.environ["CG_ENCODE_BYTES"]

@@ -466,14 +466,14 @@ int cg_encode_kv_levels(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t
         uint32_t *sym4 = reinterpret_cast<uint32_t *>(w.symbols);
         if (int rc = launch_quantize_pack(kv, kv_dt, L, T, H, D, sl, skv, st, sh, nullptr, nullptr, sym4, maxima,
                                           w.nsub, chunk_tokens, 0, s, status, nlevels, key_bins, value_bins,
-                                          (int64_t)(w.symbols_bytes / 4))) return rc;
+                                          (int64_t)(w.symbols_bytes / 4), packs_nibbles(0))) return rc;
     }
     for (int v = 0; v < nlevels; ++v) {
         const LevelOut o = {key_bins[v], value_bins[v], max_bins[v], cdf[v], lengths[v], offsets[v],
                             payload[v], payload_cap[v], status + v};
         uint8_t *symbols = w.symbols + (size_t)v * w.symbols_bytes;
         if (packed) {
-            if (int rc = code_and_compact(o, reinterpret_cast<uint32_t *>(symbols), nullptr, w, L, T, C, chunk_tokens, s, maxima, kv_dt)) return rc;
+            if (int rc = code_and_compact(o, reinterpret_cast<uint32_t *>(symbols), nullptr, w, L, T, C, chunk_tokens, s, maxima, kv_dt, packs_nibbles(0))) return rc;
         } else {
             // shapes the vector loads cannot take: one plain quantization pass per level
             clear_status_kernel<<<1, 1, 0, s>>>(status + v);

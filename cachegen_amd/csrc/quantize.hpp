@@ -284,7 +284,7 @@ __global__ __launch_bounds__(256) void quantize_pack_kernel(PackedQuantArgs a)
                     }
                     words[k] = w;
                 }
-                if (!MULTI && narrow) {
+                if (narrow) {
                     // four bits a symbol: channels 2k and 2k + 1 share word k of the unit, the even
                     // channel's four tokens in its lower half.  A saturated byte (255) becomes 15,
                     // which no symbol of such a row is: the coder gives it its meaning back.

@@ -37,7 +37,9 @@ struct TableStride {
 template <int BS>
 __device__ __forceinline__ int table_column(int c)
 {
-    return ((c & (BS / 2 - 1)) << 1) | (c / (BS / 2));
+    constexpr unsigned kHalf = BS / 2;
+    static_assert((kHalf & (kHalf - 1)) == 0, "block size must be a power of two");
+    return (int)((((unsigned)c & (kHalf - 1u)) << 1) | ((unsigned)c / kHalf));
 }
 
 // Walks i = start, start + step, ... over tables stored one after the other ([channel][lp]) and
@@ -126,14 +128,37 @@ __device__ __forceinline__ void stage_tables16(uint16_t *tab, const uint16_t *cd
     }
 }
 
+// Write the block's tables tab[entry * stride + column(lane)] to cdf[lane][entry], coalesced:
+// the tables of a block are one contiguous run of 16-bit entries, written two entries (one
+// 32-bit word) per lane and step when the run starts on a word boundary.
 template <int BS>
 __device__ __forceinline__ void write_tables16(const uint16_t *tab, uint16_t *cdf, int lp, int64_t ch0, int64_t nc)
 {
     const int64_t nvalid = (nc - ch0 < BS) ? (nc - ch0) : BS;
     const int total = (int)nvalid * lp;
+    constexpr int kS = TableStride<BS>::k16;
+    if ((reinterpret_cast<uintptr_t>(cdf) & 3u) == 0) {
+        // entry pair i = entries 2i and 2i + 1 of the run; (c, e) of the first, kept up to date
+        // by adding the step's own (c, e)
+        TableWalk w(2 * threadIdx.x, 2 * BS, lp);
+        uint32_t *out = reinterpret_cast<uint32_t *>(cdf);
+        const int pairs = total >> 1;
+        for (int i = threadIdx.x; i < pairs; i += BS, w.next(lp)) {
+            const bool wraps = w.e + 1 == lp;                           // the second entry opens the next table
+            const int c2 = wraps ? w.c + 1 : w.c, e2 = wraps ? 0 : w.e + 1;
+            const uint32_t lo = tab[__umul24(w.e, kS) + table_column<BS>(w.c)];
+            const uint32_t hi = tab[__umul24(e2, kS) + table_column<BS>(c2)];
+            out[i] = lo | (hi << 16);
+        }
+        if ((total & 1) && threadIdx.x == 0) {
+            const int c = (total - 1) / lp, e = (total - 1) - c * lp;
+            cdf[total - 1] = tab[e * kS + table_column<BS>(c)];
+        }
+        return;
+    }
     TableWalk w(threadIdx.x, BS, lp);
     for (int i = threadIdx.x; i < total; i += BS, w.next(lp)) {
-        cdf[i] = tab[w.e * TableStride<BS>::k16 + table_column<BS>(w.c)];
+        cdf[i] = tab[w.e * kS + table_column<BS>(w.c)];
     }
 }
 

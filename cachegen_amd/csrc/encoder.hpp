@@ -204,9 +204,11 @@ struct RangeEncoder {
     {
         int n;
         uint32_t t;
+        // a carry out of the 64 low bits needs 32 waiting ones: left to a branch that is next to
+        // never taken, instead of a third add in every symbol
+        uint64_t carry;
         asm("v_add_co_u32 v56, vcc, v56, %4\n\t"
-            "v_addc_co_u32 v57, vcc, 0, v57, vcc\n\t"
-            "v_addc_co_u32 v59, vcc, 0, v59, vcc\n\t"
+            "v_addc_co_u32 v57, %2, 0, v57, vcc\n\t"
             "v_add3_u32 %1, %5, v56, -1\n\t"
             "v_xor_b32 %0, %1, v56\n\t"
             "v_bitop3_b32 %1, %1, v56, %1 bitop3:0xf3\n\t"
@@ -214,9 +216,11 @@ struct RangeEncoder {
             "v_add_lshl_u32 %1, %1, %1, %0\n\t"
             "v_ffbh_u32 %1, %1\n\t"
             "v_add_u32 %0, %0, %1"
-            : "=&v"(n), "=&v"(t), "+{v[56:57]}"(tail), "+{v59}"(out_hi)
+            : "=&v"(n), "=&v"(t), "=&s"(carry), "+{v[56:57]}"(tail)
             : "v"(add), "v"(width)
             : "vcc");
+        if (__builtin_expect(carry != 0, 0))
+            asm("v_addc_co_u32 v59, %0, 0, v59, %0" : "+s"(carry), "+{v59}"(out_hi));
         return n;
     }
 

@@ -441,9 +441,10 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
             else count(CodeTag<false, kBytes>());
         }
         __syncthreads();                     // the other lane's counts are all in
-        if (id.active) normalize_column16<BS>(col, lp, lp - 1, (uint32_t)id.n);
-        __syncthreads();
-        write_tables16<BS>(tab, cdf_block, lp, ch0, a.sg.nc);
+        if (id.active) {
+            normalize_column16<BS>(col, lp, lp - 1, (uint32_t)id.n);
+            write_column16<BS>(col, cdf_block + (int64_t)tid * lp, lp);
+        }
     } else {
         stage_tables16<BS>(tab, cdf_block, lp, ch0, a.sg.nc);
         __syncthreads();

@@ -162,6 +162,33 @@ __device__ __forceinline__ void write_tables16(const uint16_t *tab, uint16_t *cd
     }
 }
 
+// Write one lane's own table, col[e * stride], e in [0, lp), to its lp consecutive 16-bit entries
+// at `mine`, two entries per 32-bit store (a table that starts off a word boundary sends its first
+// entry alone).  The lanes of a wavefront write to places lp entries apart; what this costs the
+// memory pipeline is hidden behind the vector instructions of the other wavefronts, and a store
+// takes no address arithmetic: the LDS reads and the stores use immediate offsets.
+template <int BS>
+__device__ __forceinline__ void write_column16(const uint16_t *col, uint16_t *mine, int lp)
+{
+    constexpr int kS = TableStride<BS>::k16;
+    const int first = (int)((reinterpret_cast<uintptr_t>(mine) >> 1) & 1u);
+    if (first) mine[0] = col[0];
+    const int rest = lp - first, npairs = rest >> 1;
+    const uint16_t *src = col + first * kS;
+    uint32_t *dst = reinterpret_cast<uint32_t *>(mine + first);
+    constexpr int kBatch = 8;               // pairs in flight
+    int i = 0;
+    for (; i + kBatch <= npairs; i += kBatch) {
+        uint32_t v[kBatch];
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j) v[j] = (uint32_t)src[(2 * (i + j)) * kS] | ((uint32_t)src[(2 * (i + j) + 1) * kS] << 16);
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j) dst[i + j] = v[j];
+    }
+    for (; i < npairs; ++i) dst[i] = (uint32_t)src[(2 * i) * kS] | ((uint32_t)src[(2 * i + 1) * kS] << 16);
+    if (rest & 1) mine[lp - 1] = col[(lp - 1) * kS];
+}
+
 // Running sum and normalisation of one lane's 16-bit column of counts when every one of
 // `total` tokens was counted (1 <= total <= 65535, uniform over the block): the divide of
 // cal_cdf.cu:11-14 becomes a shift or a float estimate corrected exactly.

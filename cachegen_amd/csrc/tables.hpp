@@ -128,40 +128,6 @@ __device__ __forceinline__ void stage_tables16(uint16_t *tab, const uint16_t *cd
     }
 }
 
-// Write the block's tables tab[entry * stride + column(lane)] to cdf[lane][entry], coalesced:
-// the tables of a block are one contiguous run of 16-bit entries, written two entries (one
-// 32-bit word) per lane and step when the run starts on a word boundary.
-template <int BS>
-__device__ __forceinline__ void write_tables16(const uint16_t *tab, uint16_t *cdf, int lp, int64_t ch0, int64_t nc)
-{
-    const int64_t nvalid = (nc - ch0 < BS) ? (nc - ch0) : BS;
-    const int total = (int)nvalid * lp;
-    constexpr int kS = TableStride<BS>::k16;
-    if ((reinterpret_cast<uintptr_t>(cdf) & 3u) == 0) {
-        // entry pair i = entries 2i and 2i + 1 of the run; (c, e) of the first, kept up to date
-        // by adding the step's own (c, e)
-        TableWalk w(2 * threadIdx.x, 2 * BS, lp);
-        uint32_t *out = reinterpret_cast<uint32_t *>(cdf);
-        const int pairs = total >> 1;
-        for (int i = threadIdx.x; i < pairs; i += BS, w.next(lp)) {
-            const bool wraps = w.e + 1 == lp;                           // the second entry opens the next table
-            const int c2 = wraps ? w.c + 1 : w.c, e2 = wraps ? 0 : w.e + 1;
-            const uint32_t lo = tab[__umul24(w.e, kS) + table_column<BS>(w.c)];
-            const uint32_t hi = tab[__umul24(e2, kS) + table_column<BS>(c2)];
-            out[i] = lo | (hi << 16);
-        }
-        if ((total & 1) && threadIdx.x == 0) {
-            const int c = (total - 1) / lp, e = (total - 1) - c * lp;
-            cdf[total - 1] = tab[e * kS + table_column<BS>(c)];
-        }
-        return;
-    }
-    TableWalk w(threadIdx.x, BS, lp);
-    for (int i = threadIdx.x; i < total; i += BS, w.next(lp)) {
-        cdf[i] = tab[w.e * kS + table_column<BS>(w.c)];
-    }
-}
-
 // Write one lane's own table, col[e * stride], e in [0, lp), to its lp consecutive 16-bit entries
 // at `mine`, two entries per 32-bit store (a table that starts off a word boundary sends its first
 // entry alone).  The lanes of a wavefront write to places lp entries apart; what this costs the
@@ -327,9 +293,10 @@ __global__ __launch_bounds__(BS) void calculate_cdf_kernel(CdfArgs a)
     uint16_t *dst = a.cdf + ((chunk * a.rows + row) * a.nc + ch0) * lp;
     if (PACKED) {
         __syncthreads();                     // the other lane's atomics on the shared words are done
-        if (ch < a.nc) normalize_column16<BS>(tab16 + tcol, lp, a.max_bins, (uint32_t)(t1 - t0));
-        __syncthreads();
-        write_tables16<BS>(tab16, dst, lp, ch0, a.nc);
+        if (ch < a.nc) {
+            normalize_column16<BS>(tab16 + tcol, lp, a.max_bins, (uint32_t)(t1 - t0));
+            write_column16<BS>(tab16 + tcol, dst + (int64_t)tid * lp, lp);
+        }
     } else {
         __syncthreads();
         write_tables<BS>(smem, dst, lp, ch0, a.nc);

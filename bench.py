@@ -407,14 +407,14 @@ def main():
     }
     if "valu_insts" in counters:
         # The kernel's own limit is the issue of vector instructions: one per 4 cycles per SIMD for
-        # most of them, 1024 SIMDs, at the clock the profile's GRBM_GUI_ACTIVE gives (2.3 GHz).
+        # most of them, 1024 SIMDs, at the GPU's published peak engine clock (2.4 GHz).
         insts = counters["valu_insts"]
         result["valu_issue"] = {
             "kernel": "decode_streams_kernel",
             "insts_per_launch": insts,
             "insts_per_symbol_and_lane": round(insts * 64 / (kv_bytes / 2), 1),
-            "frac_of_issue_rate": round(insts / (r["decode_ms"] * 1e-3) / (1024 * 2.3e9 / 4), 3),
-            "note": "profile counter x live duration; above 1 where cheap instructions issue in under 4 cycles",
+            "frac_of_issue_rate": round(insts / (r["decode_ms"] * 1e-3) / (1024 * 2.4e9 / 4), 3),
+            "note": "profile counter x live duration against 4 cycles per instruction at 2.4 GHz; above 1 because adds, moves and logic instructions that follow one another issue in 2",
         }
     enc_counters = measured_counters().get(args.workload, {}).get("encode_all_kernels")
     if enc_counters:

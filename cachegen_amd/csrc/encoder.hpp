@@ -103,15 +103,17 @@ struct WordWriter {
     }
 };
 
-// The coder state is the number described above plus the interval's width `span`, held
-// modulo 2^32: 0 stands for the full range 2^32 (the initial state, and any later interval
-// that is exactly a binary fraction), where floor(span * c / 2^16) is simply c << 16.
-// Renormalising by n bits maps span to span << n for E1/E2 and E3 steps alike.
+// The coder state is the number described above plus the interval's width less one,
+// `span_less_one`: the full range 2^32 (the initial state, and any later interval that is exactly
+// a binary fraction) is 2^32 - 1 there, and floor(span * c / 2^16) is the high word of
+// span_less_one * (c << 16) + (c << 16) for every span, one 64-bit multiply-add with nothing set
+// apart for the full range.  Renormalising by n bits maps span to span << n for E1/E2 and E3
+// steps alike.
 template <int BS, bool ALIGNED, bool TILE = false>
 struct RangeEncoder {
     lds_char *col;          // this lane's table column: entry e at byte e * 2 * TableStride<BS>::k16
     uint32_t smax;          // lp - 2: the largest symbol
-    uint32_t span;
+    uint32_t span_less_one;
     // the number's last 96 bits: `tail` holds the window (its lower half, called low in the
     // comments) and above it the first 32 of the bits waiting to be written, `out_hi` the rest
     // of them: 63 - room bits wait, and above them there may be a carry (0 or 1) that belongs
@@ -126,7 +128,7 @@ struct RangeEncoder {
     uint32_t plain;         // 0xFFFFFFFF while `ones` is 0, else 0: a word below it is stored the short way
     // the coded symbol's two table entries, each shifted left by 16: only ever written by
     // loads into the upper half, so that the lower halves stay zero
-    uint32_t bound_lo, bound_hi;
+    uint64_t bound_lo, bound_hi;
     WordWriter<ALIGNED, TILE> w;
 
     __device__ __forceinline__ void init(const uint16_t *column, int lp)
@@ -135,7 +137,7 @@ struct RangeEncoder {
         bound_lo = 0;
         bound_hi = 0;
         smax = (uint32_t)(lp - 2);
-        span = 0;
+        span_less_one = 0xFFFFFFFFu;
         tail = 0;
         out_hi = 0;
         room = 63;
@@ -253,23 +255,26 @@ struct RangeEncoder {
     {
         if (CLAMP) s = s < smax ? s : smax;             // keep table reads inside the table
         constexpr int kRow = 2 * TableStride<BS>::k16;
-        lds_entries_high<kRow>(col + s * kRow, bound_lo, bound_hi);
-        // the upper bound of symbol smax is 2^16 and not the table's last entry; shifted left
-        // by 16 that is 0 modulo 2^32, and T(2^16) is the span
+        // both entries into the upper halves of the lower registers of two pairs whose upper
+        // registers stay 0: the pairs are the entries shifted left by 16, as 64-bit values
+        asm volatile("ds_read_u16_d16_hi v52, %2\n\tds_read_u16_d16_hi v54, %2 offset:%3\n\ts_waitcnt lgkmcnt(0)"
+                     : "+{v[52:53]}"(bound_lo), "+{v[54:55]}"(bound_hi)
+                     : "v"(col + s * kRow), "n"(kRow));
+        // T(c) = (span * c) >> 16 = high word of span * (c << 16) = high word of
+        // span_less_one * (c << 16) + (c << 16): one 64-bit multiply-add, right for the full range
+        // (span_less_one = 2^32 - 1) as for every other span, so no case is set apart
+        uint64_t prod_lo, prod_hi;
+        asm("v_mad_u64_u32 %0, vcc, %2, v52, v[52:53]\n\tv_mad_u64_u32 %1, vcc, %2, v54, v[54:55]"
+            : "=&v"(prod_lo), "=&v"(prod_hi)
+            : "v"(span_less_one), "{v[52:53]}"(bound_lo), "{v[54:55]}"(bound_hi)
+            : "vcc");
+        const uint32_t t_lo = (uint32_t)(prod_lo >> 32);
+        // the upper bound of symbol smax is 2^16 and not the table's last entry: T(2^16) is the span
         const bool top = SENTINEL && s == smax;
-        // T(c) = (span * c) >> 16 = high word of span * (c << 16)
-        uint32_t t_lo = __umulhi(span, bound_lo);
-        uint32_t width = (top ? span : __umulhi(span, bound_hi)) - t_lo;
-        if (__builtin_expect(span == 0, 0)) {
-            // the full range: T(c) = c << 16.  The empty statement makes the compiler jump over
-            // this block when no lane needs it instead of issuing it with every lane masked off.
-            asm volatile("");
-            t_lo = bound_lo;
-            width = (top ? 0u : bound_hi) - bound_lo;
-        }
+        const uint32_t width = (top ? span_less_one + 1u : (uint32_t)(prod_hi >> 32)) - t_lo;
         const int n = add_and_count(t_lo, width);
         shift<FIRST>(n);
-        span = width << n;
+        span_less_one = (width << n) - 1u;
     }
 
     // one group of symbols is through: write a word if 32 bits are waiting

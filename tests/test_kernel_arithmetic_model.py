@@ -33,6 +33,21 @@ def bound(cdf, s, span):
     return t(c_lo), (t(c_hi) - t(c_lo)) & M32
 
 
+def bound_less_one(cdf, s, span_less_one):
+    """The same from the encoder's state, which keeps span - 1 (2^32 - 1: full range): T(c) is the
+    high word of span_less_one * (c << 16) + (c << 16), one 64-bit multiply-add (v_mad_u64_u32)
+    with no case set apart for the full range."""
+    def t(c):
+        if c == 0x10000:
+            return (span_less_one + 1) & M32               # 0 modulo 2^32 when the range is full
+        total = span_less_one * (c << 16) + (c << 16)
+        assert total < 1 << 64
+        return total >> 32
+    c_lo = cdf[s]
+    c_hi = 0x10000 if s == len(cdf) - 2 else cdf[s + 1]
+    return t(c_lo), (t(c_hi) - t(c_lo)) & M32
+
+
 def shift_count(low, high):
     n1 = clz32(low ^ high)
     z = (((low & high) | (~low & M32)) << ((n1 + 1) & 31)) & M32
@@ -45,7 +60,7 @@ def model_encode(cdf, symbols, group=8):
     a symbol adds its offset and shifts the number left by the step count; complete words leave
     once per `group` symbols through a held-back word that takes the carry, words of all ones
     being counted until the word after them shows whether a carry comes."""
-    out, low, span, nout = 0, 0, 0, 0
+    out, low, span_less_one, nout = 0, 0, M32, 0
     cache, ones, words, started = 0, 0, [], [False]
 
     def store(word):
@@ -96,12 +111,13 @@ def model_encode(cdf, symbols, group=8):
         assert out < 1 << 64
 
     for i, s in enumerate(symbols):
-        t_lo, width = bound(cdf, s, span)
+        t_lo, width = bound_less_one(cdf, s, span_less_one)
+        assert (t_lo, width) == bound(cdf, s, (span_less_one + 1) & M32)
         add_low(t_lo)
         high = (low + width - 1) & M32                     # bit 31 of low may differ from the reference's
         n1, k = shift_count(low, high)
         shift(n1 + k)
-        span = (width << (n1 + k)) & M32
+        span_less_one = ((width << (n1 + k)) - 1) & M32
         if i % group == group - 1 and nout >= 32:
             flush_word()
     add_low(0x40000000)

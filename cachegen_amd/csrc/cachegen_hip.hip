@@ -143,7 +143,7 @@ int cg_encode_fast_new(const int16_t *cdf, int lp, const int8_t *sym, int64_t nl
     const size_t shmem = (size_t)lp * (block + 2) * sizeof(uint16_t);      // TableStride<BS>::k16 per entry
     const bool aligned = aligned_to(out, 4) && o0 % 4 == 0 && o1 % 4 == 0;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const dim3 grid((unsigned)nblocks), blk(block);
+    const dim3 grid = stream_grid(a.sg, nblocks), blk(block);
     if (aligned) CG_DISPATCH_BS(block, (encode_streams_kernel<BS, true, false, false, false><<<grid, blk, shmem, st>>>(a)));
     else CG_DISPATCH_BS(block, (encode_streams_kernel<BS, false, false, false, false><<<grid, blk, shmem, st>>>(a)));
     return check_launch("encode");
@@ -334,7 +334,7 @@ int code_and_compact(const LevelOut &o, const uint32_t *sym4, const uint8_t *sym
     int64_t nblocks;
     if (int rc = make_grid(rows, C, T, chunk_tokens, w.nsub, block, a.sg, nblocks)) return rc;
     const size_t shmem = (size_t)lp * (block + 2) * sizeof(uint16_t);      // TableStride<BS>::k16 per entry
-    const dim3 grid((unsigned)nblocks), blk(block);
+    const dim3 grid = stream_grid(a.sg, nblocks), blk(block);
     // when every encoder block is exactly one tile of the scratch, the blocks leave their byte
     // counts behind and the compaction computes the stream offsets itself
     const bool fused_scan = block == kSlotTile && C % kSlotTile == 0;
@@ -532,7 +532,7 @@ int cg_decode_kv(const int16_t *cdf, int max_bins, const void *maxima, int max_d
     if (int rc = make_grid(rows, C, T, chunk_tokens, nsub, block, a.sg, nblocks)) return rc;
     const size_t shmem = decode_shmem(a.lp, block);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const dim3 grid((unsigned)nblocks);
+    const dim3 grid = stream_grid(a.sg, nblocks);
     if (out_dt == CG_DT_BF16) CG_DISPATCH_BS(block, (launch_decode_kv_log2<BS, OUT_BF16>(a, grid, shmem, s)));
     else CG_DISPATCH_BS(block, (launch_decode_kv_log2<BS, OUT_F16>(a, grid, shmem, s)));
     return check_launch("decode_kv");

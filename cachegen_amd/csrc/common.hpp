@@ -50,7 +50,8 @@ struct TokenGeom {
 __host__ __device__ inline void sub_range(const TokenGeom &g, int64_t sub, int64_t &chunk,
                                           int64_t &t0, int &n)
 {
-    chunk = sub / g.nsc;
+    // one sub-chunk per chunk (tables per 256 tokens) needs no division; otherwise both fit 32 bits
+    chunk = g.nsc == 1 ? sub : (int64_t)((uint32_t)sub / (uint32_t)g.nsc);
     const int64_t j = sub - chunk * g.nsc;
     t0 = chunk * g.S + j * kSub;
     int64_t tend = (chunk + 1) * g.S;

@@ -396,7 +396,7 @@ __global__ __launch_bounds__(BS) void decode_streams_kernel(DecodeArgs a)
     int special = 0;                   // a row maximum that is infinite or NaN
     int nsym = lp;                     // symbols the row's alphabet can hold
     if (OUT != OUT_SYMBOLS) {
-        kvi = id.row / a.L;
+        kvi = id.row >= a.L ? 1 : 0;             // 2L rows: keys, then values
         l = id.row - kvi * a.L;
         const float bins = (kvi ? a.value_bins : a.key_bins)[l];
         const float cq = floorf(bins * 0.5f) - 1.0f;
@@ -443,7 +443,7 @@ __global__ __launch_bounds__(BS) void decode_streams_kernel(DecodeArgs a)
     if (OUT == OUT_SYMBOLS) {
         s.osym = a.out_sym + id.row * a.o0 + id.t0 * a.o1 + id.ch * a.o2;
     } else {
-        const int64_t h = id.ch / a.D;
+        const int64_t h = (uint32_t)id.ch / (uint32_t)a.D;     // both fit 32 bits
         const int64_t first_row = l * a.ol + kvi * a.okv + id.t0 * a.ot;             // uniform over the block
         const uint32_t fr_lo = __builtin_amdgcn_readfirstlane((uint32_t)first_row);
         const uint32_t fr_hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)first_row >> 32));

@@ -383,7 +383,7 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
     int mode = kBytes;
     uint32_t half_shift = 0;
     if (PACKED && a.key_bins) {
-        const int64_t kvi = id.row / a.L, l = id.row - kvi * a.L;
+        const int64_t kvi = id.row >= a.L ? 1 : 0, l = id.row - kvi * a.L;       // 2L rows: keys, then values
         const float cq = floorf((kvi ? a.value_bins : a.key_bins)[l] * 0.5f) - 1.0f;
         sentinel = !(cq >= 0.0f && 2.0f * cq + 1.0f <= (float)(lp - 2));
         if (a.maxima) {
@@ -462,11 +462,11 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
     // the tile's word w * kSlotTile + t, so that the words the lanes of a wavefront write, and
     // the words the compaction reads, lie side by side
     if (TILE) {
-        // the block is exactly one tile (the host launches this form only then): blockIdx.x is
+        // the block is exactly one tile (the host launches this form only then): its number is
         // the tile, tid the stream's place in it
         enc.init(col, lp);
         enc.w.init(nullptr, 0, a.cap);
-        enc.w.init_tile(__builtin_amdgcn_make_buffer_rsrc((void *)(a.out + (int64_t)blockIdx.x * ((int64_t)kSlotTile * a.cap)), 0,
+        enc.w.init_tile(__builtin_amdgcn_make_buffer_rsrc((void *)(a.out + (int64_t)linear_block() * ((int64_t)kSlotTile * a.cap)), 0,
                                                           kSlotTile * a.cap, kBufferWord3),
                         (uint32_t)tid * 4u);
     } else if (SLOTS) {
@@ -547,7 +547,7 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
         if (tid == 0) {
             int32_t total = 0;
             for (int w = 0; w < BS / 64; ++w) total += wave_sums[w];
-            a.tile_sums[blockIdx.x] = total;                  // at most 256 streams of 256 bytes
+            a.tile_sums[linear_block()] = total;                  // at most 256 streams of 256 bytes
         }
     }
 }

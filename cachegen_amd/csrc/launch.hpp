@@ -35,7 +35,16 @@ int make_grid(int64_t rows, int64_t nc, int64_t T, int64_t S, int64_t nsub, int 
     sg.g.nsc = (int32_t)ceil_div(S, kSub);
     nblocks = nsub * rows * sg.ctiles;
     if (nblocks <= 0 || nblocks > INT_MAX) return fail(CG_ERR_ARG, "grid of %lld blocks is out of range", (long long)nblocks);
+    // the grid is three-dimensional (channel tile, row, sub-chunk), so that a block reads its place
+    // from its index instead of dividing for it
+    if (rows > 65535 || nsub > 65535)
+        return fail(CG_ERR_ARG, "%lld rows and %lld sub-chunks: at most 65535 of each in one call", (long long)rows, (long long)nsub);
     return CG_OK;
+}
+
+dim3 stream_grid(const StreamGrid &sg, int64_t nblocks)
+{
+    return dim3((unsigned)sg.ctiles, (unsigned)sg.rows, (unsigned)(nblocks / (sg.rows * sg.ctiles)));
 }
 
 // Run `launch` with the block size as a compile-time constant.
@@ -256,7 +265,7 @@ void launch_decode_log2(const DecodeArgs &a, dim3 grid, size_t shmem, hipStream_
 template <int SRC>
 int launch_decode_symbols(const DecodeArgs &a, int64_t nblocks, int block, hipStream_t stream)
 {
-    const dim3 grid((unsigned)nblocks);
+    const dim3 grid = stream_grid(a.sg, nblocks);
     const size_t shmem = decode_shmem(a.lp, block);
     CG_DISPATCH_BS(block, (launch_decode_log2<BS, SRC, OUT_SYMBOLS>(a, grid, shmem, stream)));
     return check_launch("decode");

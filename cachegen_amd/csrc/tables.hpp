@@ -319,19 +319,24 @@ struct StreamId {
     bool active;
 };
 
+// The grid is (channel tile, row, sub-chunk): a block reads its place from its index.
 template <int BS>
 __device__ __forceinline__ StreamId locate(const StreamGrid &sg)
 {
     StreamId s;
-    int64_t b = blockIdx.x;
-    const int ctile = (int)(b % sg.ctiles);
-    b /= sg.ctiles;
-    s.row = b % sg.rows;
-    s.sub = b / sg.rows;
+    s.row = blockIdx.y;
+    s.sub = blockIdx.z;
     sub_range(sg.g, s.sub, s.chunk, s.t0, s.n);
-    s.ch = (int64_t)ctile * BS + threadIdx.x;
+    s.ch = (int64_t)blockIdx.x * BS + threadIdx.x;
     s.active = s.ch < sg.nc;
     return s;
+}
+
+// The block's number in the order (sub-chunk, row, channel tile), in which tiles of the encoder's
+// scratch and their byte counts are laid out.
+__device__ __forceinline__ uint32_t linear_block()
+{
+    return (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
 }
 
 }  // namespace

@@ -7,6 +7,11 @@
  * state between calls and return CG_OK or a negative CG_ERR_* code;
  * cg_last_error() then holds a message for the calling thread.
  *
+ * The encode and decode entry points launch one block per (channel tile, row,
+ * sub-chunk of 256 tokens) on a three-dimensional grid: at most 65535 rows
+ * (layers, or 2 x layers for the *_kv functions) and 65535 sub-chunks per call,
+ * CG_ERR_ARG beyond.
+ *
  * Paths in the comments are relative to LMCache/ in the reference tree:
  *   enc_new.cu = third_party/torchac_cuda/torchac_kernel_enc_new.cu
  *   dec_new.cu = third_party/torchac_cuda/torchac_kernel_dec_new.cu

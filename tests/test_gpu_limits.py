@@ -398,3 +398,30 @@ def test_four_bit_symbol_words_give_the_same_streams_as_byte_words(dtype, chunk)
     ok = (out - src).abs() <= 0.6 * step + 1e-30             # half a step and the 16-bit rounding of the output
     sane = mx > 1e-30                                       # rows whose scale did not overflow
     assert bool((ok | ~sane.expand_as(ok)).all())
+
+
+def test_more_than_65535_rows_are_refused_and_65535_are_coded(oracle):
+    """The stream kernels run on a grid of (channel tile, row, sub-chunk): a call with more rows
+    than a grid dimension holds is refused before anything is launched, and the largest number
+    of rows that fits is coded like any other."""
+    import cachegen_amd.torchac_hip as tac
+    g = torch.Generator().manual_seed(7)
+    cdf_row = torch.tensor([0, 21845, 65535], dtype=torch.int32).to(torch.int16)
+    for nl, ok in ((65536, False), (65535, True)):
+        cdf = cdf_row.expand(nl, 1, 3).contiguous().to(DEV)
+        sym = torch.randint(0, 2, (nl, 5, 1), generator=g, dtype=torch.int8).to(DEV)
+        buf = torch.zeros((nl, 1, 16), dtype=torch.uint8, device=DEV)
+        lengths = torch.zeros((nl, 1), dtype=torch.int32, device=DEV)
+        if not ok:
+            with pytest.raises(RuntimeError, match="at most 65535"):
+                tac.encode_fast_new(cdf, sym, buf, lengths)
+            continue
+        tac.encode_fast_new(cdf, sym, buf, lengths)
+        out = torch.zeros((nl, 5, 1), dtype=torch.uint8, device=DEV)
+        tac.decode_fast_new(cdf, buf, lengths, out)
+        assert torch.equal(out.cpu(), sym.cpu().to(torch.uint8))
+        # a few rows against the oracle, the last one among them
+        for r in (0, 1, 40000, nl - 1):
+            want, n = oracle.encode_stream(cdf_row.numpy().view(np.uint16), sym[r, :, 0].cpu().numpy().astype(np.uint8))
+            assert int(lengths[r, 0]) == n
+            assert buf[r, 0, :n].cpu().numpy().tobytes() == want, r

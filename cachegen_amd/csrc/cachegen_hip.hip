@@ -21,7 +21,6 @@
 #include <climits>
 #include <cstdarg>
 #include <cstdio>
-#include <cstdlib>
 #include <cstring>
 #include <mutex>
 
@@ -309,7 +308,7 @@ struct LevelOut {
 // (encoder.py:265-292, 209-222).
 // The level's status word has been set to zero by an earlier launch of the same call.
 // maxima, max_dt: the row maxima (packed symbols only); nibbles: the quantizer packed the rows
-// of at most 15 symbols four bits a symbol (see packs_nibbles).
+// of at most 15 symbols four bits a symbol (see narrow_alphabet).
 int code_and_compact(const LevelOut &o, const uint32_t *sym4, const uint8_t *sym_bytes, const EncodeWorkspace &w,
                      int64_t L, int64_t T, int64_t C, int64_t chunk_tokens, hipStream_t s,
                      const void *maxima = nullptr, int max_dt = 0, bool nibbles = false)
@@ -382,29 +381,23 @@ int code_and_compact(const LevelOut &o, const uint32_t *sym4, const uint8_t *sym
     return check_launch("compact");
 }
 
-bool packs_nibbles(int delta_group)
-{
-    return delta_group == 0 && !getenv("CG_ENCODE_BYTES");
-}
-
 int check_kv_geometry(const char *what, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D, int64_t chunk_tokens)
 {
     if (int rc = check_dt(kv_dt, what)) return rc;
     if (L <= 0 || T <= 0 || H <= 0 || D <= 0) return fail(CG_ERR_ARG, "%s: empty input", what);
     if (chunk_tokens <= 0) return fail(CG_ERR_ARG, "%s: chunk_tokens must be positive", what);
     if (chunk_tokens > 65535) return fail(CG_ERR_ARG, "%s: at most 65535 tokens per chunk (16-bit counters)", what);
-    return CG_OK;
+    // refused here, before the first launch of the call has written anything
+    return check_grid_limits(2 * L, cg_num_subchunks(T, chunk_tokens));
 }
 
-}  // namespace
-
-extern "C" {
-
-int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D, int64_t sl,
-                 int64_t skv, int64_t st, int64_t sh, const float *key_bins, const float *value_bins,
-                 int max_bins, int64_t chunk_tokens, int delta_group, int16_t *cdf, void *maxima,
-                 int32_t *lengths, int64_t *offsets, uint8_t *payload, int64_t payload_cap,
-                 int32_t *status, void *workspace, size_t workspace_bytes, void *stream)
+// cg_encode_kv; four_bit_words: rows of at most 15 symbols travel from the quantizer to the coder
+// four bits a symbol (the product's choice), or every row a byte a symbol (the test entry point)
+int encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D, int64_t sl,
+              int64_t skv, int64_t st, int64_t sh, const float *key_bins, const float *value_bins,
+              int max_bins, int64_t chunk_tokens, int delta_group, int16_t *cdf, void *maxima,
+              int32_t *lengths, int64_t *offsets, uint8_t *payload, int64_t payload_cap,
+              int32_t *status, void *workspace, size_t workspace_bytes, void *stream, bool four_bit_words)
 {
     if (!kv || !key_bins || !value_bins || !cdf || !maxima || !lengths || !offsets || !payload || !status || !workspace)
         return fail(CG_ERR_ARG, "encode_kv: null pointer");
@@ -423,16 +416,39 @@ int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int
         return fail(CG_ERR_ARG, "encode_kv: delta groups need head sizes and strides that are multiples of 8 and a 16-byte aligned tensor");
     if (packed) {
         uint32_t *sym4 = reinterpret_cast<uint32_t *>(w.symbols);
-        // rows of at most 15 symbols travel four bits a symbol
-        const bool nibbles = packs_nibbles(delta_group);
+        const bool nibbles = four_bit_words && delta_group == 0;
         if (int rc = launch_quantize_pack(kv, kv_dt, L, T, H, D, sl, skv, st, sh, key_bins, value_bins, sym4,
                                           maxima, w.nsub, chunk_tokens, delta_group, s, status, 0, nullptr, nullptr, 0,
-                                          nibbles)) return rc;
+                                          nibbles, nullptr, max_bins + 1)) return rc;
         return code_and_compact(o, sym4, nullptr, w, L, T, C, chunk_tokens, s, maxima, kv_dt, nibbles);
     }
     clear_status_kernel<<<1, 1, 0, s>>>(status);
     if (int rc = launch_quantize(kv, kv_dt, L, T, H, D, sl, skv, st, sh, key_bins, value_bins, w.symbols, maxima, s)) return rc;
     return code_and_compact(o, nullptr, w.symbols, w, L, T, C, chunk_tokens, s);
+}
+
+}  // namespace
+
+extern "C" {
+
+int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D, int64_t sl,
+                 int64_t skv, int64_t st, int64_t sh, const float *key_bins, const float *value_bins,
+                 int max_bins, int64_t chunk_tokens, int delta_group, int16_t *cdf, void *maxima,
+                 int32_t *lengths, int64_t *offsets, uint8_t *payload, int64_t payload_cap,
+                 int32_t *status, void *workspace, size_t workspace_bytes, void *stream)
+{
+    return encode_kv(kv, kv_dt, L, T, H, D, sl, skv, st, sh, key_bins, value_bins, max_bins, chunk_tokens, delta_group,
+                     cdf, maxima, lengths, offsets, payload, payload_cap, status, workspace, workspace_bytes, stream, true);
+}
+
+int cg_test_encode_kv_byte_symbols(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D, int64_t sl,
+                                   int64_t skv, int64_t st, int64_t sh, const float *key_bins, const float *value_bins,
+                                   int max_bins, int64_t chunk_tokens, int delta_group, int16_t *cdf, void *maxima,
+                                   int32_t *lengths, int64_t *offsets, uint8_t *payload, int64_t payload_cap,
+                                   int32_t *status, void *workspace, size_t workspace_bytes, void *stream)
+{
+    return encode_kv(kv, kv_dt, L, T, H, D, sl, skv, st, sh, key_bins, value_bins, max_bins, chunk_tokens, delta_group,
+                     cdf, maxima, lengths, offsets, payload, payload_cap, status, workspace, workspace_bytes, stream, false);
 }
 
 int cg_encode_kv_levels(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D, int64_t sl,
@@ -448,10 +464,12 @@ int cg_encode_kv_levels(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t
     if (nlevels < 1 || nlevels > CG_MAX_LEVELS)
         return fail(CG_ERR_ARG, "encode_kv_levels: between 1 and %d levels, got %d", CG_MAX_LEVELS, nlevels);
     if (int rc = check_kv_geometry("encode_kv_levels", kv_dt, L, T, H, D, chunk_tokens)) return rc;
+    int lp_lv[CG_MAX_LEVELS];
     for (int v = 0; v < nlevels; ++v) {
         if (!key_bins[v] || !value_bins[v] || !cdf[v] || !lengths[v] || !offsets[v] || !payload[v])
             return fail(CG_ERR_ARG, "encode_kv_levels: null pointer for level %d", v);
         if (int rc = check_lp(max_bins[v] + 1, "encode_kv_levels")) return rc;
+        lp_lv[v] = max_bins[v] + 1;
     }
     const int64_t C = H * D;
     const EncodeWorkspace w(workspace, L, T, C, chunk_tokens, nlevels);
@@ -466,14 +484,14 @@ int cg_encode_kv_levels(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t
         uint32_t *sym4 = reinterpret_cast<uint32_t *>(w.symbols);
         if (int rc = launch_quantize_pack(kv, kv_dt, L, T, H, D, sl, skv, st, sh, nullptr, nullptr, sym4, maxima,
                                           w.nsub, chunk_tokens, 0, s, status, nlevels, key_bins, value_bins,
-                                          (int64_t)(w.symbols_bytes / 4), packs_nibbles(0))) return rc;
+                                          (int64_t)(w.symbols_bytes / 4), true, lp_lv)) return rc;
     }
     for (int v = 0; v < nlevels; ++v) {
         const LevelOut o = {key_bins[v], value_bins[v], max_bins[v], cdf[v], lengths[v], offsets[v],
                             payload[v], payload_cap[v], status + v};
         uint8_t *symbols = w.symbols + (size_t)v * w.symbols_bytes;
         if (packed) {
-            if (int rc = code_and_compact(o, reinterpret_cast<uint32_t *>(symbols), nullptr, w, L, T, C, chunk_tokens, s, maxima, kv_dt, packs_nibbles(0))) return rc;
+            if (int rc = code_and_compact(o, reinterpret_cast<uint32_t *>(symbols), nullptr, w, L, T, C, chunk_tokens, s, maxima, kv_dt, true)) return rc;
         } else {
             // shapes the vector loads cannot take: one plain quantization pass per level
             clear_status_kernel<<<1, 1, 0, s>>>(status + v);

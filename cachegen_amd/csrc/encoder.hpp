@@ -388,14 +388,15 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
         sentinel = !(cq >= 0.0f && 2.0f * cq + 1.0f <= (float)(lp - 2));
         if (a.maxima) {
             int saturates = 0;
-            if (tid < id.n) {
-                const uint32_t bits = a.maxima[id.row * a.sg.g.T + id.t0 + tid];
+            // every token row of the sub-chunk, whatever the block size
+            for (int i = tid; i < id.n; i += BS) {
+                const uint32_t bits = a.maxima[id.row * a.sg.g.T + id.t0 + i];
                 const float m = a.max_dt == CG_DT_BF16 ? load16f<CG_DT_BF16>(bits) : load16f<CG_DT_F16>(bits);
-                saturates = scale_overflows(cq, m);
+                saturates |= scale_overflows(cq, m);
             }
             if (__syncthreads_or(saturates)) sentinel = true;       // the last symbol does occur
         }
-        if (a.nibbles && narrow_alphabet(cq)) {
+        if (a.nibbles && narrow_alphabet(cq, lp)) {
             mode = sentinel ? kNibblesEscaped : kNibbles;
             if (id.active) symbols_voff = (uint32_t)(id.ch >> 1) * 4u;
             half_shift = (uint32_t)(id.ch & 1) * 16u;

@@ -24,6 +24,16 @@ int pick_block(int64_t nc, int lp)
     return block;
 }
 
+// The stream kernels run on a three-dimensional grid (channel tile, row, sub-chunk), so that a
+// block reads its place from its index instead of dividing for it: rows and sub-chunks are grid
+// dimensions and must fit one.
+int check_grid_limits(int64_t rows, int64_t nsub)
+{
+    if (rows > 65535 || nsub > 65535)
+        return fail(CG_ERR_ARG, "%lld rows and %lld sub-chunks: at most 65535 of each in one call", (long long)rows, (long long)nsub);
+    return CG_OK;
+}
+
 int make_grid(int64_t rows, int64_t nc, int64_t T, int64_t S, int64_t nsub, int block,
               StreamGrid &sg, int64_t &nblocks)
 {
@@ -35,11 +45,7 @@ int make_grid(int64_t rows, int64_t nc, int64_t T, int64_t S, int64_t nsub, int 
     sg.g.nsc = (int32_t)ceil_div(S, kSub);
     nblocks = nsub * rows * sg.ctiles;
     if (nblocks <= 0 || nblocks > INT_MAX) return fail(CG_ERR_ARG, "grid of %lld blocks is out of range", (long long)nblocks);
-    // the grid is three-dimensional (channel tile, row, sub-chunk), so that a block reads its place
-    // from its index instead of dividing for it
-    if (rows > 65535 || nsub > 65535)
-        return fail(CG_ERR_ARG, "%lld rows and %lld sub-chunks: at most 65535 of each in one call", (long long)rows, (long long)nsub);
-    return CG_OK;
+    return check_grid_limits(rows, nsub);
 }
 
 dim3 stream_grid(const StreamGrid &sg, int64_t nblocks)
@@ -190,7 +196,7 @@ int launch_quantize_pack(const void *kv, int kv_dt, int64_t L, int64_t T, int64_
                          const float *value_bins, uint32_t *sym4, void *maxima, int64_t nsub,
                          int64_t S, int delta_group, hipStream_t stream, int32_t *status, int nlevels = 0,
                          const float *const *key_bins_lv = nullptr, const float *const *value_bins_lv = nullptr,
-                         int64_t level_words = 0, bool nibbles = false)
+                         int64_t level_words = 0, bool nibbles = false, const int *lp_lv = nullptr, int lp = 0)
 {
     PackedQuantArgs a;
     memset(&a, 0, sizeof(a));
@@ -201,7 +207,9 @@ int launch_quantize_pack(const void *kv, int kv_dt, int64_t L, int64_t T, int64_
     for (int v = 0; v < nlevels; ++v) {
         a.key_bins_lv[v] = key_bins_lv[v];
         a.value_bins_lv[v] = value_bins_lv[v];
+        a.lp_lv[v] = lp_lv ? lp_lv[v] : 0;
     }
+    a.lp = lp;
     a.level_words = level_words;
     a.nibbles = nibbles ? 1 : 0;
     a.kv = static_cast<const uint16_t *>(kv);

@@ -172,6 +172,7 @@ struct PackedQuantArgs {
     int32_t nunits;         // C / 8
     int64_t nsub;
     int32_t nibbles;        // rows of at most 15 symbols are written four bits a symbol (see quantize_pack_kernel)
+    int32_t lp, lp_lv[kMaxLevels];          // table length (of every level): the symbols must also fit the table
     int32_t delta_group;    // > 0: tokens of a sub-chunk in groups of this many, see below
     TokenGeom g;
 };
@@ -191,7 +192,13 @@ __device__ __forceinline__ void clear_statuses(const PackedQuantArgs &a)
 // fifteen of them fit four bits with the value 15 to spare.  Where the caller asks for it
 // (a.nibbles) such rows are stored four bits a symbol, word w of channel pair p (channels 2p and
 // 2p + 1) of a sub-chunk at sym4[((row * nsub + sub) * 64 + w) * C + p]: half of the bytes.
-__device__ __forceinline__ bool narrow_alphabet(float maxq) { return maxq >= 0.0f && maxq <= 7.0f; }
+// The coder does not compare four-bit symbols with the table's end, so the row's alphabet must
+// also lie inside a table of `lp` entries (symbols 0 .. lp - 2); the quantizer, the table kernel
+// and the coder all decide with this one function.
+__device__ __forceinline__ bool narrow_alphabet(float maxq, int lp)
+{
+    return maxq >= 0.0f && maxq <= 7.0f && 2.0f * maxq <= (float)(lp - 2);
+}
 
 // A token row whose maximum is so small that the scale maxq / max is infinite (bfloat16 maxima
 // below about 2^-125): every non-zero value of the row saturates, to the byte 255, which the
@@ -257,7 +264,7 @@ __global__ __launch_bounds__(256) void quantize_pack_kernel(PackedQuantArgs a)
     for (int lv = 0; lv < nlevels; ++lv, out += a.level_words) {
         const float bins = MULTI ? (kvi ? a.value_bins_lv[lv] : a.key_bins_lv[lv])[l] : (kvi ? a.value_bins : a.key_bins)[l];
         const float maxq = floorf(bins * 0.5f) - 1.0f;
-        const bool narrow = a.nibbles && narrow_alphabet(maxq);
+        const bool narrow = a.nibbles && narrow_alphabet(maxq, MULTI ? a.lp_lv[lv] : a.lp);
         float factor[4];
         // rows past the end of the sub-chunk are all zero: 0 * inf = NaN -> symbol byte 0
 #pragma unroll

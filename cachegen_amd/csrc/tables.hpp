@@ -253,7 +253,7 @@ __global__ __launch_bounds__(BS) void calculate_cdf_kernel(CdfArgs a)
             bool narrow = false;                     // uniform over the block
             if (a.nibbles) {
                 const int64_t kvi = row / a.L, l = row - kvi * a.L;
-                narrow = narrow_alphabet(floorf((kvi ? a.value_bins : a.key_bins)[l] * 0.5f) - 1.0f);
+                narrow = narrow_alphabet(floorf((kvi ? a.value_bins : a.key_bins)[l] * 0.5f) - 1.0f, lp);
             }
             const int64_t column = narrow ? (ch >> 1) : ch;
             const uint32_t half_shift = narrow ? (uint32_t)(ch & 1) * 16u : 0u;

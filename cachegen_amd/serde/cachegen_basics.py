@@ -119,8 +119,38 @@ class CacheGenGPUEncoderOutput:
 
     @staticmethod
     def from_bytes(bs: bytes) -> "CacheGenGPUEncoderOutput":
+        """Reads a container written here or by the reference (cachegen_basics.py:146-156 pickles
+        the same two dataclasses under `lmcache.storage_backend.serde.cachegen_basics`).  Only the
+        globals such a pickle needs are resolved; anything else a blob names is refused, so a
+        store cannot make this call run code of its choosing."""
         with io.BytesIO(bs) as f:
-            return pickle.load(f)
+            return _ContainerUnpickler(f).load()
+
+
+def _load_storage(b: bytes):
+    # what torch.storage._load_from_bytes does, without its general unpickling
+    return torch.load(io.BytesIO(b), weights_only=True)
+
+
+class _ContainerUnpickler(pickle.Unpickler):
+    """Unpickler for CacheGenGPUEncoderOutput blobs: the two container classes under this
+    package's module path and under the reference's, and the three helpers with which torch
+    pickles a tensor (the storage's bytes are read with `weights_only=True`)."""
+
+    _CONTAINER_MODULES = ("cachegen_amd.serde.cachegen_basics", "lmcache.storage_backend.serde.cachegen_basics")
+    _CONTAINER_CLASSES = ("CacheGenGPUEncoderOutput", "CacheGenGPUBytestream", "CacheGenEncoderOutput")
+
+    def find_class(self, module, name):
+        if module in self._CONTAINER_MODULES and name in self._CONTAINER_CLASSES:
+            return globals()[name]
+        if (module, name) == ("torch._utils", "_rebuild_tensor_v2"):
+            return torch._utils._rebuild_tensor_v2
+        if (module, name) == ("torch.storage", "_load_from_bytes"):
+            return _load_storage
+        if (module, name) == ("collections", "OrderedDict"):
+            import collections
+            return collections.OrderedDict
+        raise pickle.UnpicklingError("CacheGen container: refusing to load %s.%s" % (module, name))
 
 
 # The reference's tests load the encoder output under this older name as well

@@ -155,6 +155,18 @@ int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int
                  uint8_t *payload, int64_t payload_cap, int32_t *status,
                  void *workspace, size_t workspace_bytes, void *stream);
 
+/* Test hook: cg_encode_kv with the one internal choice that has two forms switched to the other
+ * form (every row's symbols cross from the quantizer to the coder a byte a symbol; the product
+ * packs rows of at most 15 symbols four bits a symbol).  Same arguments and same results as
+ * cg_encode_kv, which is what the test that calls it checks.  No counterpart in the reference. */
+int cg_test_encode_kv_byte_symbols(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D,
+                                   int64_t sl, int64_t skv, int64_t st, int64_t sh,
+                                   const float *key_bins, const float *value_bins, int max_bins,
+                                   int64_t chunk_tokens, int delta_group,
+                                   int16_t *cdf, void *maxima, int32_t *lengths, int64_t *offsets,
+                                   uint8_t *payload, int64_t payload_cap, int32_t *status,
+                                   void *workspace, size_t workspace_bytes, void *stream);
+
 /* The same KV cache encoded at `nlevels` quantization levels from ONE read of the tensor: the
  * adaptive-streaming use of the reference, which pre-encodes every chunk at QUANT_LEVEL 1..3
  * by calling the serializer once per level (run_adaptation.py:63-72, src/utils.py:357-377).

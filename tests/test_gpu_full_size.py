@@ -123,3 +123,50 @@ def test_llama70b_table_long_chunks_round_trip():
     x, y = kv.reshape(L, 2, T, 1024).float(), out.reshape(L, 2, T, 1024).float()
     maxq = torch.stack([kb, vb], dim=1).div(2, rounding_mode="floor").sub(1)[:, :, None, None]
     assert bool(((x - y).abs() <= 0.52 * x.abs().amax(dim=-1, keepdim=True) / maxq).all())
+
+
+def test_one_table_over_the_whole_context_at_full_size(oracle):
+    """The reference's own call pattern (run_cachegen.py:53,67 hands the serializer the whole
+    context as one chunk): config 2 with ONE table per (layer, channel) over all 8192 tokens, its
+    32 sub-chunks coded against it.  Tables against an integer count on the GPU, one sub-chunk of
+    streams against the oracle's coder bit for bit, the status word against the longest stream,
+    and the round trip."""
+    from cachegen_amd import codec
+    from cachegen_amd.kvgen import make_kv
+    L, T, H, D = 32, 8192, 8, 128
+    C = H * D
+    kv = make_kv(L, T, H, D, seed=1236, device=DEV)
+    kb, vb = _bins("lmsys/longchat-7b-16k")
+    enc = codec.encode_kv(kv, kb, vb, chunk_tokens=T)
+    assert enc.cdf.shape == (1, 2 * L, C, 33) and enc.lengths.shape == (32, 2 * L, C)
+    longest = int(enc.lengths.max())
+    status = int(enc.status.item())
+    # bit 0 says exactly this: some stream outgrew the 256 bytes a stream keeps
+    assert (status & 1) == (1 if longest > 256 else 0) and (status & ~1) == 0
+    # the tables: cal_cdf.cu:29-49 from integer counts of the quantizer's own symbols
+    sym, maxima = codec.quantize_kv(kv, kb, vb)                     # uint8 [2L, T, C]
+    assert torch.equal(maxima, enc.maxima)
+    got = enc.cdf[0].view(torch.uint16).to(torch.int64)
+    for r0 in range(0, 2 * L, 8):
+        s = sym[r0:r0 + 8].to(torch.int64)                          # [8, T, C]
+        counts = torch.zeros((8, C, 33), dtype=torch.int64, device=DEV)
+        counts.scatter_add_(2, (s + 1).permute(0, 2, 1), torch.ones_like(s).permute(0, 2, 1))
+        cum = counts.cumsum(dim=2)
+        want = ((0xFFFF - 32) * cum) // T + torch.arange(33, device=DEV)
+        assert torch.equal(got[r0:r0 + 8], want), r0
+    # one sub-chunk of every row against the oracle's coder, on the GPU's tables and symbols
+    bounds = enc.sub_boundaries()
+    g = 17
+    cdf_np = enc.cdf[0].cpu().numpy().view(np.uint16)
+    sym_np = sym[:, g * 256:(g + 1) * 256].cpu().numpy()
+    padded, want_len = oracle.encode_fast_new(cdf_np, np.ascontiguousarray(sym_np))
+    assert np.array_equal(enc.lengths[g].cpu().numpy(), want_len)
+    stored = np.minimum(want_len, 256)
+    want_bytes = oracle.collect_bytes(padded, stored)
+    assert np.array_equal(enc.payload[bounds[g]:bounds[g + 1]].cpu().numpy(), want_bytes)
+    # offsets advance by the stored length
+    assert bool((enc.offsets[1:] - enc.offsets[:-1] == enc.lengths.flatten().clamp(max=256)).all())
+    if not status:
+        out = codec.decode_encoded(enc, kb, vb, fmt="vllm", out_dtype=torch.float16)
+        qsym, _ = codec.quantize_kv(out, kb, vb)
+        assert torch.equal(qsym, sym)                               # the decoder gave every symbol back

@@ -357,10 +357,9 @@ def test_carries_through_whole_words_of_ones_match_oracle(oracle):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_four_bit_symbol_words_give_the_same_streams_as_byte_words(dtype, chunk):
     """Rows of at most 15 symbols cross from the quantizer to the coder four bits a symbol.  The
-    other form (a byte a symbol, CG_ENCODE_BYTES=1) must give the same tables, streams and maxima,
+    other form (a byte a symbol, the library's test entry point) must give the same tables, streams and maxima,
     also for token rows whose scale overflows (bfloat16 maxima below 2^-125: MAX / max is
     infinite, every non-zero value saturates to the table's last symbol) and rows of zeros."""
-    import os
     codec, _ = _mods()
     torch.manual_seed(11)
     L, T, H, D = 3, 300, 4, 128
@@ -373,15 +372,10 @@ def test_four_bit_symbol_words_give_the_same_streams_as_byte_words(dtype, chunk)
     kv = kv.to(dtype).to(DEV)
     kb = torch.tensor([32.0, 16.0, 12.0])
     vb = torch.tensor([16.0, 8.0, 16.0])
-    assert "CG_ENCODE_BYTES" not in os.environ
     got = codec.encode_kv(kv, kb, vb, chunk_tokens=chunk)
     got.check()
-    os.environ["CG_ENCODE_BYTES"] = "1"
-    try:
-        ref = codec.encode_kv(kv, kb, vb, chunk_tokens=chunk)
-        ref.check()
-    finally:
-        del os.environ["CG_ENCODE_BYTES"]
+    ref = codec.encode_kv(kv, kb, vb, chunk_tokens=chunk, _entry="cg_test_encode_kv_byte_symbols")
+    ref.check()
     n = ref.total_bytes()
     assert got.total_bytes() == n
     assert torch.equal(got.cdf, ref.cdf) and torch.equal(got.lengths, ref.lengths) and torch.equal(got.offsets, ref.offsets)

@@ -91,7 +91,9 @@ def test_calculate_cdf_known_answer_on_gpu():
 # --------------------------------------------------------------------------- #
 @pytest.mark.parametrize("max_bins,nl,nt,nc,table_tokens", [
     (32, 4, 256, 1024, 256), (32, 3, 256, 96, 1500), (16, 2, 44, 33, 300), (32, 2, 1, 64, 1),
-    (64, 2, 256, 130, 256), (12, 5, 100, 7, 100)])
+    (64, 2, 256, 130, 256), (12, 5, 100, 7, 100),
+    # tables of more than 65 entries: the search that is not unrolled; more than 80 entries: blocks of 128 lanes
+    (80, 2, 256, 300, 256), (96, 2, 256, 200, 256), (128, 2, 256, 300, 700), (128, 1, 100, 64, 100), (100, 3, 31, 5, 400)])
 def test_encode_and_decode_entry_points_match_oracle(oracle, max_bins, nl, nt, nc, table_tokens):
     _, tac = gpu_mods()
     rng = np.random.default_rng(nl * 1000 + nt + nc)
@@ -184,6 +186,36 @@ def test_entry_point_errors():
 def _tables(L):
     k = torch.tensor([32.0] * (L // 2) + [16.0] * (L - L // 2))
     return k, k.clone()
+
+
+@pytest.mark.parametrize("bins,S", [((128.0, 96.0, 16.0), 256), ((96.0, 70.0, 32.0), 600), ((128.0, 128.0, 128.0), 300)])
+def test_fused_path_with_tables_up_to_the_length_limit_matches_oracle(oracle, bins, S):
+    """Tables of 97 and 129 entries (CG_MAX_LP) through cg_encode_kv and cg_decode_kv: blocks of
+    128 lanes, the search that is not unrolled, rows of 16 levels next to rows of 128."""
+    codec, _ = gpu_mods()
+    from cachegen_amd.kvgen import make_kv
+    L, T, H, D = 3, 600, 3, 64
+    kv = make_kv(L, T, H, D, seed=77, dtype=torch.float16)
+    kbins = torch.tensor(bins)
+    vbins = torch.tensor(bins[::-1])
+    enc = codec.encode_kv(kv.to(DEV), kbins.to(DEV), vbins.to(DEV), chunk_tokens=S)
+    enc.check()
+    assert enc.cdf.shape[-1] == int(max(bins)) + 1
+    flat = bits(kv).reshape(L, 2, T, H * D)
+    bounds = enc.sub_boundaries()
+    sub = 0
+    out = codec.decode_encoded(enc, kbins.to(DEV), vbins.to(DEV), fmt="vllm", out_dtype=torch.float16)
+    got_kv = bits(out).reshape(L, 2, T, H * D)
+    for ci, c0 in enumerate(range(0, T, S)):
+        c1 = min(c0 + S, T)
+        want = oracle.encode_function(np.ascontiguousarray(flat[:, :, c0:c1]), kbins.numpy(), vbins.numpy(), 0)
+        cdf, _, _, subs = enc.chunk(ci, bounds)
+        assert np.array_equal(cdf.cpu().numpy().view(np.uint16), want["cdf"])
+        for (b, l, n), (wb, wl, wn) in zip(subs, want["data_chunks"]):
+            assert n == wn and np.array_equal(l.cpu().numpy(), wl) and np.array_equal(b.cpu().numpy(), wb)
+            sub += 1
+        _, want_kv = oracle.decode_function(want, kbins.numpy(), vbins.numpy())
+        assert np.array_equal(got_kv[:, :, c0:c1], want_kv)
 
 
 @pytest.mark.parametrize("dtype,dt", [(torch.float16, 0), (torch.bfloat16, 1)])

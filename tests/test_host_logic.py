@@ -157,3 +157,97 @@ def test_decode_kv_refuses_inputs_that_do_not_have_the_geometry():
         call(offsets=offsets[:-1])
     with pytest.raises(RuntimeError, match="payload must be"):
         call(payload=payload[:0])
+
+
+def _sample_container():
+    import torch
+    from cachegen_amd.serde import cachegen_basics as B
+    g = torch.Generator().manual_seed(1)
+    chunk = B.CacheGenGPUBytestream(torch.randint(0, 256, (37,), generator=g, dtype=torch.uint8),
+                                    torch.randint(0, 9, (4, 3), generator=g, dtype=torch.int32), 7)
+    return B.CacheGenGPUEncoderOutput([chunk], torch.randint(-9, 9, (4, 3, 5), generator=g, dtype=torch.int16),
+                                      torch.randn((2, 7, 1), generator=g).to(torch.bfloat16),
+                                      torch.randn((2, 14, 1), generator=g).to(torch.float16)[:, ::2], 8, 128)
+
+
+def _same_container(a, b):
+    import torch
+    assert (a.num_heads, a.head_size, len(a.data_chunks)) == (b.num_heads, b.head_size, len(b.data_chunks))
+    for x, y in zip(a.data_chunks, b.data_chunks):
+        assert x.ntokens == y.ntokens and torch.equal(x.bytestream, y.bytestream)
+        assert torch.equal(x.bytestream_lengths, y.bytestream_lengths)
+    for f in ("cdf", "max_tensors_key", "max_tensors_value"):
+        assert a[f].dtype == b[f].dtype and torch.equal(a[f], b[f])
+
+
+def test_container_reads_a_blob_pickled_under_the_references_module_path():
+    """The reference pickles `lmcache.storage_backend.serde.cachegen_basics.CacheGenGPUEncoderOutput`
+    (cachegen_basics.py:133-156).  Such a blob is made here by pickling this package's own classes
+    while they claim that module path; no reference code is imported."""
+    from cachegen_amd.serde import cachegen_basics as B
+    obj = _sample_container()
+    mine = obj.to_bytes()
+    _same_container(B.CacheGenGPUEncoderOutput.from_bytes(mine), obj)
+
+    # pickle with the classes temporarily claiming the reference's module path
+    saved = {c: c.__module__ for c in (B.CacheGenGPUEncoderOutput, B.CacheGenGPUBytestream)}
+    import sys
+    import types
+    ref_name = "lmcache.storage_backend.serde.cachegen_basics"
+    # pickle checks that module.name is the object it writes: empty stand-in modules, for the
+    # length of the dump only
+    parts = ref_name.split(".")
+    names = [".".join(parts[:i + 1]) for i in range(len(parts))]
+    assert not any(n in sys.modules for n in names)
+    try:
+        for n in names:
+            sys.modules[n] = types.ModuleType(n)
+        sys.modules[ref_name].CacheGenGPUEncoderOutput = B.CacheGenGPUEncoderOutput
+        sys.modules[ref_name].CacheGenGPUBytestream = B.CacheGenGPUBytestream
+        for c in saved:
+            c.__module__ = ref_name
+        theirs = obj.to_bytes()
+    finally:
+        for c, m in saved.items():
+            c.__module__ = m
+        for n in names:
+            sys.modules.pop(n, None)
+    assert ref_name.encode() in theirs and b"cachegen_amd" not in theirs
+    assert ref_name not in sys.modules
+    _same_container(B.CacheGenGPUEncoderOutput.from_bytes(theirs), obj)
+
+
+def test_container_refuses_any_other_global():
+    import pickle
+    import pytest
+    from cachegen_amd.serde import cachegen_basics as B
+    for evil in (pickle.dumps(print), pickle.dumps(__import__("os").system),
+                 b"cbuiltins\neval\n(V1+1\ntR."):
+        with pytest.raises(pickle.UnpicklingError, match="refusing to load"):
+            B.CacheGenGPUEncoderOutput.from_bytes(evil)
+
+
+def test_built_kernels_keep_their_register_budget():
+    """The stream kernels need eight wavefronts per SIMD and no scratch memory; the build writes
+    the compiler's figures beside the library and refuses a library that breaks a budget.  This
+    reads the figures of the library the other tests load."""
+    import json
+    import os
+    from cachegen_amd import build
+    assert os.path.exists(build.RESOURCES), "build the library with cachegen_amd.build.build_library()"
+    assert os.path.getmtime(build.RESOURCES) >= os.path.getmtime(build.LIBRARY) - 120, "resource report older than the library"
+    with open(build.RESOURCES) as f:
+        resources = json.load(f)
+    build.check_budgets(resources)
+    fused = resources["encode_streams_kernel<256, true, true, true, true, true>"]
+    assert fused["vgprs"] <= 64 and fused["scratch"] == 0 and fused["occupancy"] == 8
+    # the check does fail when a kernel crosses the line
+    import pytest
+    broken = dict(resources)
+    broken["encode_streams_kernel<256, true, true, true, true, true>"] = dict(fused, vgprs=72, occupancy=7)
+    with pytest.raises(RuntimeError, match="budget 8"):
+        build.check_budgets(broken)
+    spilled = dict(resources)
+    spilled["compact_streams_kernel<true>"] = dict(resources["compact_streams_kernel<true>"], scratch=16)
+    with pytest.raises(RuntimeError, match="scratch"):
+        build.check_budgets(spilled)

@@ -35,17 +35,24 @@ def test_static_scan_equals_the_workspace_scan_on_two_calls_in_a_row():
     big = torch.randint(0, 257, (64 * 1024 * 9 + 321,), generator=g, dtype=torch.int32).to(DEV)     # 289 tiles, ragged
     small = torch.randint(0, 257, (2048 * 3 + 7,), generator=g, dtype=torch.int32).to(DEV)          # 4 tiles
     tiny = torch.randint(0, 257, (100,), generator=g, dtype=torch.int32).to(DEV)                    # a single tile
-    want = [_scan_with_workspace(lib, t) for t in (big, small, tiny)]
+    # more than 16384 lengths: like `big` it takes the three-launch scan that uses the built-in
+    # array, of which it overwrites only the first 21 of the 290 sums `big` leaves there
+    mid = torch.randint(0, 257, (2048 * 20 + 33,), generator=g, dtype=torch.int32).to(DEV)
+    inputs = (big, small, tiny, mid)
+    want = [_scan_with_workspace(lib, t) for t in inputs]
     # outputs exist before the calls under test: nothing is allocated between or inside them
-    outs = [torch.full((t.numel() + 1,), -1, dtype=torch.int64, device=DEV) for t in (big, small, tiny)]
+    outs = [torch.full((t.numel() + 1,), -1, dtype=torch.int64, device=DEV) for t in inputs]
     torch.cuda.synchronize()
     before = torch.cuda.memory_allocated()
+    free_before = torch.cuda.mem_get_info()[0]       # the driver's own count: a hipMalloc inside the library would show here
     _scan_static(lib, big, outs[0])
     _scan_static(lib, small, outs[1])
     _scan_static(lib, tiny, outs[2])
+    _scan_static(lib, mid, outs[3])
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == before
-    for got, ref, src in zip(outs, want, (big, small, tiny)):
+    assert torch.cuda.mem_get_info()[0] == free_before
+    for got, ref, src in zip(outs, want, inputs):
         assert torch.equal(got, ref)
         host = np.concatenate([[0], np.cumsum(src.cpu().numpy().astype(np.int64))])
         assert np.array_equal(got.cpu().numpy(), host)

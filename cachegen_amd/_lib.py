@@ -32,8 +32,8 @@ SIGNATURES = {
     "cg_encode_kv_workspace": (_SZ, [_I64, _I64, _I64, _I64]),
     "cg_encode_kv": (_INT, [_P, _INT, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _P, _P, _INT, _I64, _INT,
                             _P, _P, _P, _P, _P, _I64, _P, _P, _SZ, _P]),
-    "cg_test_encode_kv_byte_symbols": (_INT, [_P, _INT, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _P, _P, _INT, _I64, _INT,
-                                              _P, _P, _P, _P, _P, _I64, _P, _P, _SZ, _P]),
+    "cg_test_encode_kv": (_INT, [_P, _INT, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _P, _P, _INT, _I64, _INT,
+                                 _P, _P, _P, _P, _P, _I64, _P, _P, _SZ, _P, _INT]),
     "cg_encode_kv_levels_workspace": (_SZ, [_I64, _I64, _I64, _I64, _INT]),
     "cg_encode_kv_levels": (_INT, [_P, _INT, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _INT, _P, _P, _P, _I64,
                                    _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),

@@ -33,6 +33,7 @@ OCCUPANCY_BUDGETS = [
     (r"^decode_streams_kernel<", 8),
     (r"^compact_streams_kernel<", 8),
     (r"^quantize_pack_kernel<[01], (true|false), 2, false>", 8),                # up to 1024 channels, one level
+    (r"^quantize_tables_kernel<[01], (true|false), [12], (9|17|33)>", 4),       # two blocks of eight wavefronts per compute unit
 ]
 
 

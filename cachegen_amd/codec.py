@@ -111,14 +111,14 @@ def encode_workspace_bytes(num_layers, num_tokens, num_channels, chunk_tokens):
 
 
 def encode_kv(kv, key_bins, value_bins, chunk_tokens=None, fmt="vllm", max_bins=None,
-              workspace=None, out: Optional[EncodedKV] = None, delta_group=0, _entry="cg_encode_kv"):
+              workspace=None, out: Optional[EncodedKV] = None, delta_group=0, _test_flags=None):
     """kv: fp16/bf16 GPU tensor [L,2,T,H,D] (fmt "vllm") or [L,2,H,T,D] ("huggingface").
     key_bins / value_bins: float32 GPU tensors [L].  chunk_tokens: tokens per table
     (default: all T, i.e. one `to_bytes` call).  `workspace` (uint8, GPU) and `out`
     (a previous result of the same geometry) let a caller reuse memory.  delta_group > 0
     switches on delta-against-anchor quantization in token groups of that size (an extension:
-    the reference codec has none); decode with the same value.  `_entry` names the library entry
-    point (the tests call the library's test hook, which has the same signature, through it)."""
+    the reference codec has none); decode with the same value.  `_test_flags` (tests only) goes to the
+    library's test entry point, which takes the same arguments and must give the same results."""
     if not kv.is_cuda:
         raise RuntimeError("KV tensor should be on GPU")
     if kv.dtype not in _DT:
@@ -168,12 +168,15 @@ def encode_kv(kv, key_bins, value_bins, chunk_tokens=None, fmt="vllm", max_bins=
                 out.delta_group) != (L, T, H, D, S, max_bins, int(delta_group)):
             raise RuntimeError("encode_kv: `out` was made for another geometry")
     with torch.cuda.device(dev):
-        _lib.check(getattr(lib, _entry)(
-            kv.data_ptr(), _DT[kv.dtype], L, T, H, D, sl, skv, st, sh,
-            key_bins.data_ptr(), value_bins.data_ptr(), max_bins, S, int(delta_group),
-            out.cdf.data_ptr(), out.maxima.data_ptr(), out.lengths.data_ptr(), out.offsets.data_ptr(),
-            out.payload.data_ptr(), out.payload.numel(), out.status.data_ptr(),
-            workspace.data_ptr(), workspace.numel(), _stream()))
+        args = (kv.data_ptr(), _DT[kv.dtype], L, T, H, D, sl, skv, st, sh,
+                key_bins.data_ptr(), value_bins.data_ptr(), max_bins, S, int(delta_group),
+                out.cdf.data_ptr(), out.maxima.data_ptr(), out.lengths.data_ptr(), out.offsets.data_ptr(),
+                out.payload.data_ptr(), out.payload.numel(), out.status.data_ptr(),
+                workspace.data_ptr(), workspace.numel(), _stream())
+        if _test_flags is None:
+            _lib.check(lib.cg_encode_kv(*args))
+        else:
+            _lib.check(lib.cg_test_encode_kv(*args, int(_test_flags)))
     return out
 
 

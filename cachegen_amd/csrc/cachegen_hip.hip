@@ -22,6 +22,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <atomic>
 #include <mutex>
 
 #include "cachegen_hip.h"
@@ -34,6 +35,7 @@
 #include "common.hpp"
 #include "quantize.hpp"
 #include "tables.hpp"
+#include "quantize_tables.hpp"
 #include "encoder.hpp"
 #include "decoder.hpp"
 #include "scan_compact.hpp"
@@ -309,9 +311,10 @@ struct LevelOut {
 // The level's status word has been set to zero by an earlier launch of the same call.
 // maxima, max_dt: the row maxima (packed symbols only); nibbles: the quantizer packed the rows
 // of at most 15 symbols four bits a symbol (see narrow_alphabet).
+// tables_ready: the tables were written by an earlier launch of the call (quantize_tables_kernel).
 int code_and_compact(const LevelOut &o, const uint32_t *sym4, const uint8_t *sym_bytes, const EncodeWorkspace &w,
                      int64_t L, int64_t T, int64_t C, int64_t chunk_tokens, hipStream_t s,
-                     const void *maxima = nullptr, int max_dt = 0, bool nibbles = false)
+                     const void *maxima = nullptr, int max_dt = 0, bool nibbles = false, bool tables_ready = false)
 {
     const int64_t rows = 2 * L;
     const int lp = o.max_bins + 1;
@@ -345,7 +348,10 @@ int code_and_compact(const LevelOut &o, const uint32_t *sym4, const uint8_t *sym
         a.nibbles = nibbles ? 1 : 0;
         a.maxima = static_cast<const uint16_t *>(maxima);
         a.max_dt = max_dt;
-        if (chunk_tokens <= kSub) {
+        if (tables_ready) {
+            if (fused_scan) encode_streams_kernel<kSlotTile, true, true, false, true, true><<<grid, blk, shmem, s>>>(a);
+            else CG_DISPATCH_BS(block, (encode_streams_kernel<BS, true, true, false, true><<<grid, blk, shmem, s>>>(a)));
+        } else if (chunk_tokens <= kSub) {
             // one sub-chunk per chunk: the encoder builds the tables itself
             if (fused_scan) encode_streams_kernel<kSlotTile, true, true, true, true, true><<<grid, blk, shmem, s>>>(a);
             else CG_DISPATCH_BS(block, (encode_streams_kernel<BS, true, true, true, true><<<grid, blk, shmem, s>>>(a)));
@@ -391,14 +397,15 @@ int check_kv_geometry(const char *what, int kv_dt, int64_t L, int64_t T, int64_t
     return check_grid_limits(2 * L, cg_num_subchunks(T, chunk_tokens));
 }
 
-// cg_encode_kv; four_bit_words: rows of at most 15 symbols travel from the quantizer to the coder
-// four bits a symbol (the product's choice), or every row a byte a symbol (the test entry point)
+// cg_encode_kv.  `flags` (CG_TEST_*, 0 from cg_encode_kv) switch the internal choices that have
+// two forms to the form the call would not take by itself; the results are the same.
 int encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D, int64_t sl,
               int64_t skv, int64_t st, int64_t sh, const float *key_bins, const float *value_bins,
               int max_bins, int64_t chunk_tokens, int delta_group, int16_t *cdf, void *maxima,
               int32_t *lengths, int64_t *offsets, uint8_t *payload, int64_t payload_cap,
-              int32_t *status, void *workspace, size_t workspace_bytes, void *stream, bool four_bit_words)
+              int32_t *status, void *workspace, size_t workspace_bytes, void *stream, int flags)
 {
+    const bool four_bit_words = !(flags & CG_TEST_BYTE_SYMBOLS);
     if (!kv || !key_bins || !value_bins || !cdf || !maxima || !lengths || !offsets || !payload || !status || !workspace)
         return fail(CG_ERR_ARG, "encode_kv: null pointer");
     if (int rc = check_kv_geometry("encode_kv", kv_dt, L, T, H, D, chunk_tokens)) return rc;
@@ -417,6 +424,20 @@ int encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_
     if (packed) {
         uint32_t *sym4 = reinterpret_cast<uint32_t *>(w.symbols);
         const bool nibbles = four_bit_words && delta_group == 0;
+        // The quantizer counts the symbols as it makes them and writes the tables, where the
+        // tables fit its LDS and there are chunks enough to fill the GPU; the coder then only codes.
+        QuantTablesShape shape;
+        const int64_t nchunks = cg_num_chunks(T, chunk_tokens);
+        const bool enough_blocks = (flags & CG_TEST_TABLES_IN_QUANTIZER) || 2 * L * nchunks >= kQuantTablesMinBlocks;
+        // the table builder addresses a chunk's token rows with a 32-bit offset from the chunk's first
+        const int64_t reach = chunk_tokens < T ? chunk_tokens : T;
+        const bool addressable = st >= 0 && sh >= 0 && ((H - 1) * sh + (D - 1) + (reach - 1) * st) * 2 + 16 <= 0xFFFFFFF0ll;
+        if (delta_group == 0 && !(flags & CG_TEST_TABLES_IN_CODER) && enough_blocks && addressable &&
+            quantize_tables_shape(C / 8, max_bins + 1, sh == D, shape)) {
+            if (int rc = launch_quantize_tables(kv, kv_dt, L, T, H, D, sl, skv, st, sh, key_bins, value_bins, sym4, maxima,
+                                                reinterpret_cast<uint16_t *>(cdf), w.nsub, chunk_tokens, nibbles, status, shape, s)) return rc;
+            return code_and_compact(o, sym4, nullptr, w, L, T, C, chunk_tokens, s, maxima, kv_dt, nibbles, true);
+        }
         if (int rc = launch_quantize_pack(kv, kv_dt, L, T, H, D, sl, skv, st, sh, key_bins, value_bins, sym4,
                                           maxima, w.nsub, chunk_tokens, delta_group, s, status, 0, nullptr, nullptr, 0,
                                           nibbles, nullptr, max_bins + 1)) return rc;
@@ -438,17 +459,17 @@ int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int
                  int32_t *status, void *workspace, size_t workspace_bytes, void *stream)
 {
     return encode_kv(kv, kv_dt, L, T, H, D, sl, skv, st, sh, key_bins, value_bins, max_bins, chunk_tokens, delta_group,
-                     cdf, maxima, lengths, offsets, payload, payload_cap, status, workspace, workspace_bytes, stream, true);
+                     cdf, maxima, lengths, offsets, payload, payload_cap, status, workspace, workspace_bytes, stream, 0);
 }
 
-int cg_test_encode_kv_byte_symbols(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D, int64_t sl,
-                                   int64_t skv, int64_t st, int64_t sh, const float *key_bins, const float *value_bins,
-                                   int max_bins, int64_t chunk_tokens, int delta_group, int16_t *cdf, void *maxima,
-                                   int32_t *lengths, int64_t *offsets, uint8_t *payload, int64_t payload_cap,
-                                   int32_t *status, void *workspace, size_t workspace_bytes, void *stream)
+int cg_test_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D, int64_t sl,
+                      int64_t skv, int64_t st, int64_t sh, const float *key_bins, const float *value_bins,
+                      int max_bins, int64_t chunk_tokens, int delta_group, int16_t *cdf, void *maxima,
+                      int32_t *lengths, int64_t *offsets, uint8_t *payload, int64_t payload_cap,
+                      int32_t *status, void *workspace, size_t workspace_bytes, void *stream, int flags)
 {
     return encode_kv(kv, kv_dt, L, T, H, D, sl, skv, st, sh, key_bins, value_bins, max_bins, chunk_tokens, delta_group,
-                     cdf, maxima, lengths, offsets, payload, payload_cap, status, workspace, workspace_bytes, stream, false);
+                     cdf, maxima, lengths, offsets, payload, payload_cap, status, workspace, workspace_bytes, stream, flags);
 }
 
 int cg_encode_kv_levels(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D, int64_t sl,

@@ -120,6 +120,12 @@ __device__ __forceinline__ uint32_t scale_span(uint32_t sh, uint32_t sl, uint32_
     return mul24(sh, c) + (mul24(sl, c) >> 16);
 }
 
+// A compile-time flag as a value, for generic lambdas.
+template <bool B>
+struct BoolTag {
+    static constexpr bool value = B;
+};
+
 // Fourth word of a buffer descriptor for raw (untyped, unswizzled) access on gfx9-family
 // GPUs: 32-bit data format, everything else off.
 constexpr int kBufferWord3 = 0x00020000;

@@ -319,11 +319,6 @@ struct EncodeArgs {
 };
 
 
-template <bool B>
-struct BoolTag {
-    static constexpr bool value = B;
-};
-
 // How a packed word holds its four symbols: kBytes, a byte each (any value; kept inside the
 // table where it is used); kNibbles, four bits each, every one a table symbol; kNibblesEscaped,
 // four bits each where 15 stands for a saturated byte, i.e. the table's last symbol.
@@ -452,7 +447,10 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
             write_column16<BS>(col, cdf_block + (int64_t)tid * lp, lp);
         }
     } else {
-        stage_tables16<BS>(tab, cdf_block, lp, ch0, a.sg.nc);
+        // packed symbols: every lane copies its own table (the transposed copy costs a division
+        // and a dozen instructions an entry; this one costs the coder under one a symbol)
+        if (!PACKED) stage_tables16<BS>(tab, cdf_block, lp, ch0, a.sg.nc);
+        else if (id.active) stage_column16_stride<TableStride<BS>::k16>(col, cdf_block + (int64_t)tid * lp, lp);
         __syncthreads();
     }
     if (!id.active) return;

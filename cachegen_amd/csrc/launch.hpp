@@ -242,6 +242,110 @@ int launch_quantize_pack(const void *kv, int kv_dt, int64_t L, int64_t T, int64_
     return check_launch("quantize_pack");
 }
 
+// The quantizer that also builds the tables (quantize_tables_kernel): which of its forms takes a tensor of `nunits` units of 8 channels and tables of `lp` entries,
+// if any.
+struct QuantTablesShape {
+    int nu, lp;
+    size_t lds;
+};
+
+constexpr size_t kMaxLdsPerBlock = 160 * 1024;      // gfx950
+// fewer (row, chunk) blocks than this leave compute units idle: the two-kernel form is used instead
+constexpr int64_t kQuantTablesMinBlocks = 512;
+
+bool quantize_tables_shape(int64_t nunits, int lp, bool heads_contiguous, QuantTablesShape &shape)
+{
+    // 2048 channels: only tensors whose heads follow one another (the other form runs out of registers)
+    const int nu = nunits <= 64 ? 1 : nunits <= 128 ? 2 : (nunits <= 256 && heads_contiguous) ? 4 : 0;
+    if (!nu || (lp != 9 && lp != 17 && lp != 33 && lp != 65)) return false;
+    shape.nu = nu;
+    shape.lp = lp;
+    shape.lds = (size_t)nu * 4 * lp * 256;
+    return shape.lds <= kMaxLdsPerBlock;
+}
+
+template <int DT, bool HC, int NU, int LP>
+int launch_quantize_tables_form(const QuantTablesArgs &a, dim3 grid, hipStream_t stream)
+{
+    typedef CountLayout<NU, LP> Layout;
+    if (Layout::kBytes > (int)kMaxLdsPerBlock) return fail(CG_ERR_ARG, "quantize_tables: tables do not fit the LDS");
+    if (Layout::kBytes > 64 * 1024) {
+        // more than 64 KiB of dynamic LDS has to be asked for, once per device
+        static std::atomic<uint64_t> asked{0};
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return fail(CG_ERR_LAUNCH, "quantize_tables: hipGetDevice");
+        if (!(asked.load(std::memory_order_relaxed) >> dev & 1)) {
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&quantize_tables_kernel<DT, HC, NU, LP>),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, Layout::kBytes);
+            if (e != hipSuccess) return fail(CG_ERR_LAUNCH, "quantize_tables: hipFuncSetAttribute: %s", hipGetErrorString(e));
+            asked.fetch_or(1ull << dev, std::memory_order_relaxed);
+        }
+    }
+    quantize_tables_kernel<DT, HC, NU, LP><<<grid, dim3(QuantTablesBlock<NU>::kThreads), Layout::kBytes, stream>>>(a);
+    return check_launch("quantize_tables");
+}
+
+template <int DT, bool HC, int LP>
+int launch_quantize_tables_nu(const QuantTablesArgs &a, const QuantTablesShape &shape, dim3 grid, hipStream_t stream)
+{
+    if (shape.nu == 1) return launch_quantize_tables_form<DT, HC, 1, LP>(a, grid, stream);
+    if (shape.nu == 2) return launch_quantize_tables_form<DT, HC, 2, LP>(a, grid, stream);
+    if (HC && LP <= 33) return launch_quantize_tables_form<DT, true, 4, (LP <= 33 ? LP : 33)>(a, grid, stream);
+    return fail(CG_ERR_ARG, "quantize_tables: shape not built");
+}
+
+template <int DT, bool HC>
+int launch_quantize_tables_shape(const QuantTablesArgs &a, const QuantTablesShape &shape, dim3 grid, hipStream_t stream)
+{
+    switch (shape.lp) {
+    case 9: return launch_quantize_tables_nu<DT, HC, 9>(a, shape, grid, stream);
+    case 17: return launch_quantize_tables_nu<DT, HC, 17>(a, shape, grid, stream);
+    case 33: return launch_quantize_tables_nu<DT, HC, 33>(a, shape, grid, stream);
+    case 65: return launch_quantize_tables_nu<DT, HC, 65>(a, shape, grid, stream);
+    }
+    return fail(CG_ERR_ARG, "quantize_tables: shape not built");
+}
+
+// Quantization, row maxima, packed symbols and the tables of every chunk in one launch.
+int launch_quantize_tables(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D,
+                           int64_t sl, int64_t skv, int64_t st, int64_t sh, const float *key_bins,
+                           const float *value_bins, uint32_t *sym4, void *maxima, uint16_t *cdf, int64_t nsub, int64_t S,
+                           bool nibbles, int32_t *status,
+                           const QuantTablesShape &shape, hipStream_t stream)
+{
+    QuantTablesArgs a;
+    memset(&a, 0, sizeof(a));
+    a.kv = static_cast<const uint16_t *>(kv);
+    a.L = L;
+    a.sl = sl;
+    a.skv = skv;
+    a.st = st;
+    a.sh = sh;
+    a.D = (int32_t)D;
+    a.key_bins = key_bins;
+    a.value_bins = value_bins;
+    a.status = status;
+    a.sym4 = sym4;
+    a.maxima = static_cast<uint16_t *>(maxima);
+    a.cdf = cdf;
+    a.nunits = (int32_t)(H * D / 8);
+    a.nsub = nsub;
+    a.nibbles = nibbles ? 1 : 0;
+    a.g.T = T;
+    a.g.S = S;
+    a.g.nsc = (int32_t)ceil_div(S, kSub);
+    const int64_t nchunks = ceil_div(T, S);
+    if (nchunks > INT_MAX || 2 * L > 65535) return fail(CG_ERR_ARG, "quantize_tables: grid out of range");
+    const dim3 grid((unsigned)nchunks, (unsigned)(2 * L));
+    const bool contiguous = (sh == D);
+    if (kv_dt == CG_DT_F16) {
+        if (contiguous) return launch_quantize_tables_shape<CG_DT_F16, true>(a, shape, grid, stream);
+        return launch_quantize_tables_shape<CG_DT_F16, false>(a, shape, grid, stream);
+    }
+    if (contiguous) return launch_quantize_tables_shape<CG_DT_BF16, true>(a, shape, grid, stream);
+    return launch_quantize_tables_shape<CG_DT_BF16, false>(a, shape, grid, stream);
+}
+
 // Describe the readable byte window [bytes, bytes + nbytes) to the bit reader, which
 // loads aligned words at 32-bit offsets from the window's 4-byte-aligned base.
 int set_byte_window(DecodeArgs &a, const uint8_t *bytes, int64_t nbytes, const char *what)

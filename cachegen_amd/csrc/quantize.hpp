@@ -209,6 +209,78 @@ __device__ __forceinline__ bool scale_overflows(float maxq, float row_max)
     return row_max != 0.0f && (__float_as_uint(__fdiv_rn(maxq, row_max)) & 0x7FFFFFFFu) == 0x7F800000u;
 }
 
+// The 4 x NU units (128-bit loads of 8 channels) that one lane holds of four consecutive token
+// rows, and the rows' maxima (largest sign-stripped 16-bit pattern, over the whole wavefront).
+// Rows j >= nvalid and units past the last channel are zeros.
+template <bool HEADS_CONTIGUOUS, int NU>
+__device__ __forceinline__ void load_four_rows(const uint16_t *base, int64_t st, int64_t sh, int D, int nunits,
+                                               int nvalid, int lane, uint4 (&regs)[4][NU], uint32_t (&max_bits)[4])
+{
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        uint32_t m = 0;
+#pragma unroll
+        for (int i = 0; i < NU; ++i) {
+            regs[j][i] = make_uint4(0, 0, 0, 0);
+            const int u = lane + 64 * i;
+            if (j < nvalid && u < nunits) {
+                const int e = u * 8;
+                int64_t off;
+                if (HEADS_CONTIGUOUS) off = e;
+                else { const int h = e / D; off = (int64_t)h * sh + (e - h * D); }
+                // read once and never again: loaded past the caches' keep-for-reuse policy
+                typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+                const u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base + j * st + off));
+                regs[j][i] = make_uint4(t.x, t.y, t.z, t.w);
+                m = pk_max_u16(m, regs[j][i].x & 0x7FFF7FFFu);
+                m = pk_max_u16(m, regs[j][i].y & 0x7FFF7FFFu);
+                m = pk_max_u16(m, regs[j][i].z & 0x7FFF7FFFu);
+                m = pk_max_u16(m, regs[j][i].w & 0x7FFF7FFFu);
+            }
+        }
+        m = (m & 0xFFFFu) > (m >> 16) ? (m & 0xFFFFu) : (m >> 16);
+        max_bits[j] = wave_max_u32(m);
+    }
+}
+
+// The symbols of one unit: word k holds channel k's four tokens, a byte each.
+template <int DT>
+__device__ __forceinline__ void quantize_unit(const uint4 (&r)[4], const float (&factor)[4], float maxq, uint32_t (&words)[8])
+{
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        uint32_t w = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t src = k < 2 ? r[j].x : k < 4 ? r[j].y : k < 6 ? r[j].z : r[j].w;
+            const uint32_t bits = (k & 1) ? (src >> 16) : (src & 0xFFFFu);
+            const float v = load16f<DT>(bits);
+            const float s = __fadd_rn(__fmul_rn(v, factor[j]), maxq);
+            // the conversion itself rounds to nearest even, turns a NaN (0 * inf of an
+            // all-zero row) and anything negative into 0 and saturates at 255: the
+            // round-half-even, int8 cast and NaN rule of encoder.py:56-57 in one step
+            w = __builtin_amdgcn_cvt_pk_u8_f32(s, (uint32_t)j, w);
+        }
+        words[k] = w;
+    }
+}
+
+// Four bits a symbol: channels 2k and 2k + 1 share word k of the unit, the even channel's four
+// tokens in its lower half.  A saturated byte (255) becomes 15, which no symbol of such a row is:
+// the coder gives it its meaning back.
+__device__ __forceinline__ uint4 pack_four_bit_words(const uint32_t (&words)[8])
+{
+    uint32_t half[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        uint32_t e = words[2 * k] & 0x0F0F0F0Fu, o = words[2 * k + 1] & 0x0F0F0F0Fu;
+        e |= e >> 4;                                    // bytes 0 and 2 hold two symbols each
+        o |= o >> 4;
+        half[k] = __builtin_amdgcn_perm(o, e, 0x06040200u);          // e.b0, e.b2, o.b0, o.b2
+    }
+    return make_uint4(half[0], half[1], half[2], half[3]);
+}
+
 template <int DT, bool HEADS_CONTIGUOUS, int NU, bool MULTI = false>
 __global__ __launch_bounds__(256) void quantize_pack_kernel(PackedQuantArgs a)
 {
@@ -229,33 +301,13 @@ __global__ __launch_bounds__(256) void quantize_pack_kernel(PackedQuantArgs a)
     const uint16_t *base = a.kv + l * a.sl + kvi * a.skv + (t0 + tt0) * a.st;
 
     uint4 regs[4][NU];
+    uint32_t max_bits[4];
     float rowmax[4];
+    load_four_rows<HEADS_CONTIGUOUS, NU>(base, a.st, a.sh, a.D, a.nunits, nvalid, lane, regs, max_bits);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        uint32_t m = 0;
-#pragma unroll
-        for (int i = 0; i < NU; ++i) {
-            regs[j][i] = make_uint4(0, 0, 0, 0);
-            const int u = lane + 64 * i;
-            if (j < nvalid && u < a.nunits) {
-                const int e = u * 8;
-                int64_t off;
-                if (HEADS_CONTIGUOUS) off = e;
-                else { const int h = e / a.D; off = (int64_t)h * a.sh + (e - h * a.D); }
-                // read once and never again: loaded past the caches' keep-for-reuse policy
-                typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-                const u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base + j * a.st + off));
-                regs[j][i] = make_uint4(t.x, t.y, t.z, t.w);
-                m = pk_max_u16(m, regs[j][i].x & 0x7FFF7FFFu);
-                m = pk_max_u16(m, regs[j][i].y & 0x7FFF7FFFu);
-                m = pk_max_u16(m, regs[j][i].z & 0x7FFF7FFFu);
-                m = pk_max_u16(m, regs[j][i].w & 0x7FFF7FFFu);
-            }
-        }
-        m = (m & 0xFFFFu) > (m >> 16) ? (m & 0xFFFFu) : (m >> 16);
-        m = wave_max_u32(m);
-        if (j < nvalid && lane == 0) a.maxima[row * a.g.T + t0 + tt0 + j] = (uint16_t)m;
-        rowmax[j] = load16f<DT>(m);
+        if (j < nvalid && lane == 0) a.maxima[row * a.g.T + t0 + tt0 + j] = (uint16_t)max_bits[j];
+        rowmax[j] = load16f<DT>(max_bits[j]);
     }
 
     const int64_t C = (int64_t)a.nunits * 8;
@@ -274,36 +326,10 @@ __global__ __launch_bounds__(256) void quantize_pack_kernel(PackedQuantArgs a)
             const int u = lane + 64 * i;
             if (u < a.nunits) {
                 uint32_t words[8];
-#pragma unroll
-                for (int k = 0; k < 8; ++k) {
-                    uint32_t w = 0;
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const uint32_t src = k < 2 ? regs[j][i].x : k < 4 ? regs[j][i].y
-                                           : k < 6 ? regs[j][i].z : regs[j][i].w;
-                        const uint32_t bits = (k & 1) ? (src >> 16) : (src & 0xFFFFu);
-                        const float v = load16f<DT>(bits);
-                        const float s = __fadd_rn(__fmul_rn(v, factor[j]), maxq);
-                        // the conversion itself rounds to nearest even, turns a NaN (0 * inf of an
-                        // all-zero row) and anything negative into 0 and saturates at 255: the
-                        // round-half-even, int8 cast and NaN rule of encoder.py:56-57 in one step
-                        w = __builtin_amdgcn_cvt_pk_u8_f32(s, (uint32_t)j, w);
-                    }
-                    words[k] = w;
-                }
+                const uint4 r[4] = {regs[0][i], regs[1][i], regs[2][i], regs[3][i]};
+                quantize_unit<DT>(r, factor, maxq, words);
                 if (narrow) {
-                    // four bits a symbol: channels 2k and 2k + 1 share word k of the unit, the even
-                    // channel's four tokens in its lower half.  A saturated byte (255) becomes 15,
-                    // which no symbol of such a row is: the coder gives it its meaning back.
-                    uint32_t half[4];
-#pragma unroll
-                    for (int k = 0; k < 4; ++k) {
-                        uint32_t e = words[2 * k] & 0x0F0F0F0Fu, o = words[2 * k + 1] & 0x0F0F0F0Fu;
-                        e |= e >> 4;                                    // bytes 0 and 2 hold two symbols each
-                        o |= o >> 4;
-                        half[k] = __builtin_amdgcn_perm(o, e, 0x06040200u);          // e.b0, e.b2, o.b0, o.b2
-                    }
-                    *reinterpret_cast<uint4 *>(out + (int64_t)u * 4) = make_uint4(half[0], half[1], half[2], half[3]);
+                    *reinterpret_cast<uint4 *>(out + (int64_t)u * 4) = pack_four_bit_words(words);
                 } else {
                     uint4 *dst = reinterpret_cast<uint4 *>(out + (int64_t)u * 8);
                     dst[0] = make_uint4(words[0], words[1], words[2], words[3]);

@@ -128,15 +128,31 @@ __device__ __forceinline__ void stage_tables16(uint16_t *tab, const uint16_t *cd
     }
 }
 
-// Write one lane's own table, col[e * stride], e in [0, lp), to its lp consecutive 16-bit entries
+// Copy one lane's own table (lp consecutive 16-bit entries at `mine`) into its LDS column
+// col[e * kS]: loads and LDS writes on immediate offsets, sixteen loads in flight; the lanes of a
+// wavefront read neighbouring tables, so every cache line is fetched once.
+template <int kS>
+__device__ __forceinline__ void stage_column16_stride(uint16_t *col, const uint16_t *mine, int lp)
+{
+    constexpr int kBatch = 16;
+    for (int e0 = 0; e0 < lp; e0 += kBatch) {
+        uint16_t v[kBatch];
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j) v[j] = e0 + j < lp ? mine[e0 + j] : (uint16_t)0;
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j)
+            if (e0 + j < lp) col[(e0 + j) * kS] = v[j];
+    }
+}
+
+// Write one lane's own table, col[e * kS], e in [0, lp), to its lp consecutive 16-bit entries
 // at `mine`, two entries per 32-bit store (a table that starts off a word boundary sends its first
 // entry alone).  The lanes of a wavefront write to places lp entries apart; what this costs the
 // memory pipeline is hidden behind the vector instructions of the other wavefronts, and a store
 // takes no address arithmetic: the LDS reads and the stores use immediate offsets.
-template <int BS>
-__device__ __forceinline__ void write_column16(const uint16_t *col, uint16_t *mine, int lp)
+template <int kS>
+__device__ __forceinline__ void write_column16_stride(const uint16_t *col, uint16_t *mine, int lp)
 {
-    constexpr int kS = TableStride<BS>::k16;
     const int first = (int)((reinterpret_cast<uintptr_t>(mine) >> 1) & 1u);
     if (first) mine[0] = col[0];
     const int rest = lp - first, npairs = rest >> 1;
@@ -155,13 +171,12 @@ __device__ __forceinline__ void write_column16(const uint16_t *col, uint16_t *mi
     if (rest & 1) mine[lp - 1] = col[(lp - 1) * kS];
 }
 
-// Running sum and normalisation of one lane's 16-bit column of counts when every one of
+// Running sum and normalisation of one lane's 16-bit column of counts (col[e * kS]) when every one of
 // `total` tokens was counted (1 <= total <= 65535, uniform over the block): the divide of
 // cal_cdf.cu:11-14 becomes a shift or a float estimate corrected exactly.
-template <int BS>
-__device__ __forceinline__ void normalize_column16(uint16_t *col, int lp, int max_bins, uint32_t total)
+template <int kS>
+__device__ __forceinline__ void normalize_column16_stride(uint16_t *col, int lp, int max_bins, uint32_t total)
 {
-    constexpr int kS = TableStride<BS>::k16;
     const uint32_t scale = 0xFFFFu - (uint32_t)max_bins;
     uint32_t running = 0;
     if ((total & (total - 1)) == 0) {
@@ -182,6 +197,18 @@ __device__ __forceinline__ void normalize_column16(uint16_t *col, int lp, int ma
             col[i * kS] = (uint16_t)(q + (uint32_t)i);
         }
     }
+}
+
+// The same two for a block's tables with the row stride of TableStride<BS>.
+template <int BS>
+__device__ __forceinline__ void write_column16(const uint16_t *col, uint16_t *mine, int lp)
+{
+    write_column16_stride<TableStride<BS>::k16>(col, mine, lp);
+}
+template <int BS>
+__device__ __forceinline__ void normalize_column16(uint16_t *col, int lp, int max_bins, uint32_t total)
+{
+    normalize_column16_stride<TableStride<BS>::k16>(col, lp, max_bins, total);
 }
 
 struct CdfArgs {

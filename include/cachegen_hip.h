@@ -155,17 +155,26 @@ int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int
                  uint8_t *payload, int64_t payload_cap, int32_t *status,
                  void *workspace, size_t workspace_bytes, void *stream);
 
-/* Test hook: cg_encode_kv with the one internal choice that has two forms switched to the other
- * form (every row's symbols cross from the quantizer to the coder a byte a symbol; the product
- * packs rows of at most 15 symbols four bits a symbol).  Same arguments and same results as
- * cg_encode_kv, which is what the test that calls it checks.  No counterpart in the reference. */
-int cg_test_encode_kv_byte_symbols(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D,
-                                   int64_t sl, int64_t skv, int64_t st, int64_t sh,
-                                   const float *key_bins, const float *value_bins, int max_bins,
-                                   int64_t chunk_tokens, int delta_group,
-                                   int16_t *cdf, void *maxima, int32_t *lengths, int64_t *offsets,
-                                   uint8_t *payload, int64_t payload_cap, int32_t *status,
-                                   void *workspace, size_t workspace_bytes, void *stream);
+/* Test hook: cg_encode_kv with the internal choices that have two forms switched by `flags` to
+ * the form the call would not take by itself.  Same arguments and the same results as
+ * cg_encode_kv, which is what the tests that call it check.  No counterpart in the reference.
+ * CG_TEST_BYTE_SYMBOLS          every row's symbols cross from the quantizer to the coder a byte a
+ *                               symbol (cg_encode_kv packs rows of at most 15 symbols four bits a symbol)
+ * CG_TEST_TABLES_IN_QUANTIZER   the quantizer counts the symbols and writes the tables, however few
+ *                               chunks the call has (cg_encode_kv does so from 512 (row, chunk) pairs on,
+ *                               where the tables of all channels fit the LDS of one block)
+ * CG_TEST_TABLES_IN_CODER       never: the coder (one table per sub-chunk) or a separate pass over
+ *                               the symbols (longer chunks) builds the tables */
+#define CG_TEST_BYTE_SYMBOLS 1
+#define CG_TEST_TABLES_IN_QUANTIZER 2
+#define CG_TEST_TABLES_IN_CODER 4
+int cg_test_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D,
+                      int64_t sl, int64_t skv, int64_t st, int64_t sh,
+                      const float *key_bins, const float *value_bins, int max_bins,
+                      int64_t chunk_tokens, int delta_group,
+                      int16_t *cdf, void *maxima, int32_t *lengths, int64_t *offsets,
+                      uint8_t *payload, int64_t payload_cap, int32_t *status,
+                      void *workspace, size_t workspace_bytes, void *stream, int flags);
 
 /* The same KV cache encoded at `nlevels` quantization levels from ONE read of the tensor: the
  * adaptive-streaming use of the reference, which pre-encodes every chunk at QUANT_LEVEL 1..3

@@ -374,7 +374,7 @@ def test_four_bit_symbol_words_give_the_same_streams_as_byte_words(dtype, chunk)
     vb = torch.tensor([16.0, 8.0, 16.0])
     got = codec.encode_kv(kv, kb, vb, chunk_tokens=chunk)
     got.check()
-    ref = codec.encode_kv(kv, kb, vb, chunk_tokens=chunk, _entry="cg_test_encode_kv_byte_symbols")
+    ref = codec.encode_kv(kv, kb, vb, chunk_tokens=chunk, _test_flags=1)          # CG_TEST_BYTE_SYMBOLS
     ref.check()
     n = ref.total_bytes()
     assert got.total_bytes() == n

@@ -171,6 +171,7 @@ int cg_decode_fast_new(const int16_t *cdf, int lp, const uint8_t *padded, int64_
     a.o0 = o0;
     a.o1 = o1;
     a.o2 = o2;
+    a.last_round_first = 0xFFFFFFFFu;     // one sub-chunk: a single round of blocks
     int64_t nblocks;
     if (int rc = make_grid(nl, nc, nt, nt, 1, block, a.sg, nblocks)) return rc;
     return launch_decode_symbols<SRC_PADDED>(a, nblocks, block, static_cast<hipStream_t>(stream));
@@ -195,6 +196,7 @@ int cg_decode_fast_prefsum(const int16_t *cdf, int lp, const uint8_t *bytes, int
     a.o0 = o0;
     a.o1 = o1;
     a.o2 = o2;
+    a.last_round_first = 0xFFFFFFFFu;     // one sub-chunk: a single round of blocks
     int64_t nblocks;
     if (int rc = make_grid(nl, nc, nt, nt, 1, block, a.sg, nblocks)) return rc;
     return launch_decode_symbols<SRC_PREFIX>(a, nblocks, block, static_cast<hipStream_t>(stream));
@@ -572,6 +574,10 @@ int cg_decode_kv(const int16_t *cdf, int max_bins, const void *maxima, int max_d
     const size_t shmem = decode_shmem(a.lp, block);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const dim3 grid = stream_grid(a.sg, nblocks);
+    // the blocks that are resident together at the launch's end (32 wavefronts per compute unit
+    // where registers and LDS allow it, which they do for tables of up to 33 entries)
+    const int64_t resident = (int64_t)compute_units() * (2048 / block);
+    a.last_round_first = (uint32_t)(nblocks > resident ? nblocks - resident : 0);
     if (out_dt == CG_DT_BF16) CG_DISPATCH_BS(block, (launch_decode_kv_log2<BS, OUT_BF16>(a, grid, shmem, s)));
     else CG_DISPATCH_BS(block, (launch_decode_kv_log2<BS, OUT_F16>(a, grid, shmem, s)));
     return check_launch("decode_kv");

@@ -139,6 +139,9 @@ struct DecodeArgs {
     int32_t max_dt;
     int32_t delta_group;        // > 0: rows that are not the first of their group hold deltas
     const float *key_bins, *value_bins;
+    // blocks from this one on (in launch order) start when no block is left to take a finished
+    // one's place: see decode_lane
+    uint32_t last_round_first;
     StreamGrid sg;
 };
 
@@ -312,8 +315,16 @@ __device__ __forceinline__ void decode_symbol(const DecodeArgs &a, DecodeLane &s
     s.off = s.rd.shift_in(s.off, n);
 }
 
+// last_round: the block is one of the launch's last, after which nothing takes the place of a
+// finished wavefront.  A wavefront alone on its SIMD cannot go faster than its own dependent
+// chain, so the launch ends when the wavefront that started last has run its 256 symbols at that
+// pace, while the SIMDs idle more and more (measured: the last 130 us of a 550 us launch, about
+// 50 us of issue time lost).  The hardware issues from the oldest wavefront first, which finishes
+// the most advanced wavefronts first and leaves the least advanced for the end; these blocks
+// raise their wavefronts' priority by the work they have left instead, so that the wavefronts of
+// a SIMD finish closer together.
 template <int BS, int LOG2, int OUT, int SKIP, bool SAFE>
-__device__ __forceinline__ void decode_lane(const DecodeArgs &a, DecodeLane &s, int lp, int n, lds_f32 *rmp)
+__device__ __forceinline__ void decode_lane(const DecodeArgs &a, DecodeLane &s, int lp, int n, lds_f32 *rmp, bool last_round)
 {
     int nsteps = 0;
     if (LOG2 < 0)
@@ -331,6 +342,13 @@ __device__ __forceinline__ void decode_lane(const DecodeArgs &a, DecodeLane &s, 
     // group, only when a symbol has left it short of bits
     constexpr int kGroup = kSymbolsPerTopUp;
     for (int i0 = 0; i0 < n; i0 += kGroup, rmp += kGroup) {
+        if (last_round && (i0 & 63) == 0) {             // uniform over the wavefront
+            const int left = (n - i0) >> 6;
+            if (left >= 3) __builtin_amdgcn_s_setprio(3);
+            else if (left == 2) __builtin_amdgcn_s_setprio(2);
+            else if (left == 1) __builtin_amdgcn_s_setprio(1);
+            else __builtin_amdgcn_s_setprio(0);
+        }
         // the maxima of the group's token rows (the array is padded to a whole group)
         float rm[kGroup];
 #pragma unroll
@@ -455,9 +473,10 @@ __global__ __launch_bounds__(BS) void decode_streams_kernel(DecodeArgs a)
 
     // all three conditions are uniform over the block
     const bool safe = OUT == OUT_SYMBOLS || LOG2 < 0 || special || a.delta_group > 0 || nsym > lp - 2;
-    if (safe) decode_lane<BS, LOG2, OUT, 0, true>(a, s, lp, id.n, rmp);
-    else if (LOG2 > 1 && nsym <= (1 << (LOG2 > 1 ? LOG2 - 1 : 0))) decode_lane<BS, LOG2, OUT, 1, false>(a, s, lp, id.n, rmp);
-    else decode_lane<BS, LOG2, OUT, 0, false>(a, s, lp, id.n, rmp);
+    const bool last_round = linear_block() >= a.last_round_first;
+    if (safe) decode_lane<BS, LOG2, OUT, 0, true>(a, s, lp, id.n, rmp, last_round);
+    else if (LOG2 > 1 && nsym <= (1 << (LOG2 > 1 ? LOG2 - 1 : 0))) decode_lane<BS, LOG2, OUT, 1, false>(a, s, lp, id.n, rmp, last_round);
+    else decode_lane<BS, LOG2, OUT, 0, false>(a, s, lp, id.n, rmp, last_round);
 }
 
 }  // namespace

@@ -346,6 +346,20 @@ int launch_quantize_tables(const void *kv, int kv_dt, int64_t L, int64_t T, int6
     return launch_quantize_tables_shape<CG_DT_BF16, false>(a, shape, grid, stream);
 }
 
+// Compute units of the current device (asked once per device).
+int compute_units()
+{
+    static std::atomic<int> known[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    int n = known[dev].load(std::memory_order_relaxed);
+    if (!n) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        known[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
+
 // Describe the readable byte window [bytes, bytes + nbytes) to the bit reader, which
 // loads aligned words at 32-bit offsets from the window's 4-byte-aligned base.
 int set_byte_window(DecodeArgs &a, const uint8_t *bytes, int64_t nbytes, const char *what)

@@ -155,7 +155,7 @@ def measured_counters():
         return json.load(f)
 
 
-def run_workload(name, steps, warmup, fmt="vllm", copy_probe=False, keep=False, ramp_ms=0.0):
+def run_workload(name, steps, warmup, fmt="vllm", copy_probe=False, keep=False, ramp_ms=0.0, sample_clock=False):
     """Encode + decode of one workload, timed with HIP events on the launching stream.
     Returns a dict of figures (and, with keep=True, the tensors for further use)."""
     import torch
@@ -212,6 +212,22 @@ def run_workload(name, steps, warmup, fmt="vllm", copy_probe=False, keep=False, 
         ev[i][2].record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
+    clock = None
+    if sample_clock:
+        # The engine clock these steps run at: the same steps once more, untimed, with one idle
+        # wavefront on a side stream that reads the shader clock against the 100 MHz counter over
+        # their whole length.  (Not during the timed steps: a resident wavefront leaves its SIMD one
+        # slot short, and that compute unit's blocks then hold up the end of every launch: +2 to 4 %.)
+        from cachegen_amd import issue_probe
+        side = torch.cuda.Stream()
+        issue_probe.clock_window_start(max(200, int(0.9 * wall * 1e6)), side.cuda_stream)
+        for i in range(steps):
+            encode()
+            decode()
+        torch.cuda.synchronize()
+        mhz, window_us = issue_probe.clock_window_result()
+        clock = {"engine_clock_mhz": round(mhz, 1), "window_us": round(window_us, 1),
+                 "what": "average over a repetition of the timed steps (%d steps, %.1f ms)" % (steps, wall * 1e3)}
 
     enc_ms = sorted(e[0].elapsed_time(e[1]) for e in ev)
     dec_ms = sorted(e[1].elapsed_time(e[2]) for e in ev)
@@ -259,6 +275,7 @@ def run_workload(name, steps, warmup, fmt="vllm", copy_probe=False, keep=False, 
         "payload_bytes": payload, "algorithmic_bytes": ab,
         "round_trip_within_half_step": verified if not status else None,
         "streams_cut_at_256_bytes": bool(status & 1), "longest_stream_bytes": int(enc.lengths.max().item()),
+        "clock": clock,
     }
     if 256 < chunk < T:
         # streaming case: latency of decoding one chunk on its own
@@ -386,6 +403,8 @@ def main():
     ap.add_argument("--cpu-sample-tokens", type=int, default=8192)
     ap.add_argument("--fmt", default="vllm", choices=["vllm", "huggingface"],
                     help="layout of the KV tensor: [L,2,T,H,D] (vllm, the metric's layout) or [L,2,H,T,D]")
+    ap.add_argument("--no-issue-probe", action="store_true",
+                    help="skip the engine-clock sampler and the instruction-issue calibration (valu_issue)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one plain device copy of the KV tensor (calibrates rocprofv3 byte counters)")
     args = ap.parse_args()
@@ -402,7 +421,7 @@ def main():
     torch.cuda.set_device(0)
     fmt = args.fmt
     r = run_workload(args.workload, args.steps, args.warmup, fmt=fmt, copy_probe=args.copy_probe, keep=True,
-                     ramp_ms=args.clock_ramp_ms)
+                     ramp_ms=args.clock_ramp_ms, sample_clock=not args.no_issue_probe)
     kept = r.pop("_keep")
     ab = r["algorithmic_bytes"]
     kv_bytes = r["kv_bytes"]
@@ -454,17 +473,39 @@ def main():
             "avg_launch_ms": round(r["decode_ms"], 4),
         },
     }
-    if "valu_insts" in counters:
-        # The kernel's own limit is the issue of vector instructions: one per 4 cycles per SIMD for
-        # most of them, 1024 SIMDs, at the GPU's published peak engine clock (2.4 GHz).
+    if "valu_insts" in counters and not args.no_issue_probe:
+        # The decoder's own limit is the issue of vector instructions.  Its instruction count per
+        # launch (the committed profile's SQ_INSTS_VALU) is priced with what this GPU issues, measured
+        # now by the calibration probe (cachegen_amd/csrc/issue_probe.hip): cycles per wave64
+        # instruction of the cheap class (adds, logic, right shifts, moves, float add/multiply on
+        # registers) and of all others, at the engine clock sampled while the timed steps ran.
+        from cachegen_amd import issue_probe
+        cal = issue_probe.calibrate()
         insts = counters["valu_insts"]
+        cheap = counters.get("cheap_class_fraction", 11.0 / 38.0)
+        simds = torch.cuda.get_device_properties(0).multi_processor_count * 4
+        mhz = (r.get("clock") or {}).get("engine_clock_mhz") or cal["decoder_symbol"]["clock_mhz"]
+        per_simd = insts / simds
+        two_class = cheap * cal["cheap"]["cycles_per_instruction"] + (1.0 - cheap) * cal["full"]["cycles_per_instruction"]
+        bound_ms = per_simd * two_class / (mhz * 1e3)
+        seq_ms = per_simd * cal["decoder_symbol"]["cycles_per_instruction"] / (mhz * 1e3)
         result["valu_issue"] = {
             "kernel": "decode_streams_kernel",
             "insts_per_launch": insts,
             "insts_per_symbol_and_lane": round(insts * 64 / (kv_bytes / 2), 1),
-            "frac_of_issue_rate": round(insts / (r["decode_ms"] * 1e-3) / (1024 * 2.4e9 / 4), 3),
-            "note": "profile counter x live duration against 4 cycles per instruction at 2.4 GHz; above 1 because adds, moves and logic instructions that follow one another issue in 2",
+            "cheap_class_fraction": round(cheap, 3),
+            "calibration": cal,
+            "engine_clock_mhz_during_timed_steps": mhz,
+            "issue_time_ms_two_class": round(bound_ms, 4),
+            "frac_of_issue_rate": round(bound_ms / r["decode_ms"], 3),
+            "issue_time_ms_same_sequence_in_probe": round(seq_ms, 4),
+            "frac_of_probe_sequence_rate": round(seq_ms / r["decode_ms"], 3),
+            "note": "instruction count of the committed profile x cycles per instruction measured now by the probe "
+                    "(two classes; and the decoder's own symbol sequence issued from the probe) / engine clock "
+                    "sampled during the timed steps / live decode time",
         }
+    if r.get("clock"):
+        result["clock"] = r["clock"]
     enc_counters = measured_counters().get(args.workload, {}).get("encode_all_kernels")
     if enc_counters:
         result["encode_traffic"] = {

@@ -16,6 +16,9 @@ _ROOT = os.path.dirname(_PKG)
 SOURCE = os.path.join(_PKG, "csrc", "cachegen_hip.hip")
 LIBRARY = os.path.join(_PKG, "lib", "libcachegen_hip.so")
 RESOURCES = os.path.join(_PKG, "lib", "kernel_resources.json")
+# the calibration probe bench.py prices the decoder's instruction count with (not part of the codec)
+PROBE_SOURCE = os.path.join(_PKG, "csrc", "issue_probe.hip")
+PROBE_LIBRARY = os.path.join(_PKG, "lib", "libcachegen_probe.so")
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
@@ -100,5 +103,18 @@ def build_library(verbose=False):
     return LIBRARY
 
 
+def build_probe():
+    """Compile csrc/issue_probe.hip into lib/libcachegen_probe.so."""
+    os.makedirs(os.path.dirname(PROBE_LIBRARY), exist_ok=True)
+    hipcc = os.environ.get("HIPCC", "hipcc")
+    cmd = [hipcc, "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-o", PROBE_LIBRARY, PROBE_SOURCE]
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + " ".join(cmd) + "\n" + res.stdout)
+    return PROBE_LIBRARY
+
+
 if __name__ == "__main__":
     print(build_library(verbose=True))
+    print(build_probe())

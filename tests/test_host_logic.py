@@ -251,3 +251,10 @@ def test_built_kernels_keep_their_register_budget():
     spilled["compact_streams_kernel<true>"] = dict(resources["compact_streams_kernel<true>"], scratch=16)
     with pytest.raises(RuntimeError, match="scratch"):
         build.check_budgets(spilled)
+
+
+def test_probe_library_loads_and_exports_its_entry_points():
+    from cachegen_amd import issue_probe
+    h = issue_probe.lib()
+    for name in ("cg_probe_issue_rate", "cg_probe_clock_start", "cg_probe_clock_result"):
+        assert hasattr(h, name)

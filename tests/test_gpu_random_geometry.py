@@ -51,7 +51,20 @@ def test_random_wide_case_matches_oracle(oracle, seed):
     run_cases(oracle, seed, 2, True)
 
 
-def run_cases(oracle, seed, ncases, wide):
+@pytest.mark.parametrize("seed", range(12, 24))
+def test_random_case_with_tables_built_by_the_quantizer(oracle, seed):
+    """The same sweep with the form of cg_encode_kv that small calls do not take by themselves
+    forced through the library's test entry point (CG_TEST_TABLES_IN_QUANTIZER); shapes the form
+    does not cover (table lengths other than 9, 17, 33, 65; more than 2048 channels) fall back."""
+    run_cases(oracle, seed, 4, False, flags=2)
+
+
+@pytest.mark.parametrize("seed", range(106, 110))
+def test_random_wide_case_with_tables_built_by_the_quantizer(oracle, seed):
+    run_cases(oracle, seed, 2, True, flags=2)
+
+
+def run_cases(oracle, seed, ncases, wide, flags=None):
     from cachegen_amd import codec
     from cachegen_amd.kvgen import make_kv
     rng = np.random.default_rng(9000 + seed)
@@ -82,7 +95,7 @@ def run_cases(oracle, seed, ncases, wide):
             big[:, :, 1:1 + T] = dev_kv
             src = big[:, :, 1:1 + T]
         kbt, vbt = torch.from_numpy(kb), torch.from_numpy(vb)
-        enc = codec.encode_kv(src, kbt, vbt, chunk_tokens=S, fmt=fmt)
+        enc = codec.encode_kv(src, kbt, vbt, chunk_tokens=S, fmt=fmt, _test_flags=flags)
         enc.check()
         bounds = enc.sub_boundaries()
         out_dtype = [torch.float16, torch.bfloat16][int(rng.integers(0, 2))]

@@ -479,7 +479,9 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
     auto code = [&](auto tag) {
         constexpr bool SENTINEL = decltype(tag)::SENTINEL;
         constexpr int MODE = decltype(tag)::MODE;
-        constexpr bool CLAMP = MODE == kBytes;
+        // a byte can lie outside the table only where the table's last symbol can occur at all
+        // (a saturated row, a table shorter than the row's alphabet, symbols handed in by a caller)
+        constexpr bool CLAMP = MODE == kBytes && SENTINEL;
         const uint32_t smax = (uint32_t)(lp - 2);
         if (PACKED) {
             for (int h = 0; h * 32 < nwords; ++h) {

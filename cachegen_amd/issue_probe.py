@@ -61,3 +61,8 @@ def clock_window_result():
     if rc:
         raise RuntimeError("cg_probe_clock_result: hipError %d" % rc)
     return mhz.value, us.value
+
+
+if __name__ == "__main__":
+    import json
+    print(json.dumps(calibrate(), indent=1))

@@ -56,12 +56,13 @@ def _overflowing_kv(T, C=64):
     return kv
 
 
-def test_stream_longer_than_256_bytes_is_reported(oracle):
+@pytest.mark.parametrize("flags", [None, 2])       # 2: the tables come from the quantizer's own counters (65280 tokens in one block)
+def test_stream_longer_than_256_bytes_is_reported(oracle, flags):
     codec, _ = _mods()
     T = 65280
     kv = _overflowing_kv(T)
     bins = torch.tensor([32.0])
-    enc = codec.encode_kv(kv.to(DEV), bins, bins, chunk_tokens=T)
+    enc = codec.encode_kv(kv.to(DEV), bins, bins, chunk_tokens=T, _test_flags=flags)
     with pytest.raises(RuntimeError, match="exceeded 256 bytes"):
         enc.check()
     lengths = enc.lengths.cpu().numpy()

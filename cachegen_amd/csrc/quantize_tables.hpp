@@ -1,5 +1,6 @@
 // Part of the CacheGen KV codec library for MI355X (gfx950); included by cachegen_hip.hip, which
-// is the one translation unit.  Row maxima and tables in one read-only pass over the tensor.
+// is the one translation unit.  Quantization, row maxima, packed symbols and the tables of every
+// chunk in one pass over the tensor.
 //
 // Paths in the comments are relative to LMCache/ in the reference tree:
 //   enc_new.cu = third_party/torchac_cuda/torchac_kernel_enc_new.cu

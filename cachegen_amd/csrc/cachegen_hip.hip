@@ -430,14 +430,28 @@ int encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_
         // tables fit its LDS and there are chunks enough to fill the GPU; the coder then only codes.
         QuantTablesShape shape;
         const int64_t nchunks = cg_num_chunks(T, chunk_tokens);
-        const bool enough_blocks = (flags & CG_TEST_TABLES_IN_QUANTIZER) || 2 * L * nchunks >= kQuantTablesMinBlocks;
+        const int64_t reach = chunk_tokens < T ? chunk_tokens : T;       // tokens of the longest chunk
+        // Few (row, chunk) pairs but long chunks (one table over a whole context): the chunks are
+        // cut into parts of whole sub-chunks, a block each, whose counters are summed in memory
+        // (in the stream slots of the workspace, which nothing uses before the coder runs).
+        int64_t part_tokens = 0;
+        if ((flags & CG_TEST_SPLIT_CHUNKS) && reach > kSub) part_tokens = kSub;
+        else if (2 * L * nchunks < kQuantTablesMinBlocks && reach > kSub) {
+            const int64_t want = ceil_div(kQuantTablesPartBlocks, 2 * L * nchunks);     // parts per chunk
+            part_tokens = reach / want / kSub * kSub;
+            if (part_tokens < kSub) part_tokens = kSub;
+        }
+        const int64_t nparts = part_tokens ? ceil_div(reach, part_tokens) : 1;
+        const bool enough_blocks = (flags & CG_TEST_TABLES_IN_QUANTIZER) || 2 * L * nchunks * nparts >= kQuantTablesMinBlocks;
         // the table builder addresses a chunk's token rows with a 32-bit offset from the chunk's first
-        const int64_t reach = chunk_tokens < T ? chunk_tokens : T;
         const bool addressable = st >= 0 && sh >= 0 && ((H - 1) * sh + (D - 1) + (reach - 1) * st) * 2 + 16 <= 0xFFFFFFF0ll;
         if (delta_group == 0 && !(flags & CG_TEST_TABLES_IN_CODER) && enough_blocks && addressable &&
             quantize_tables_shape(C / 8, max_bins + 1, sh == D, shape)) {
+            const size_t slots_bytes = (size_t)w.ntiles * kSlotTile * kStreamCap;
+            if (nparts > 1 && (size_t)nchunks * 2 * L * shape.lds > slots_bytes) part_tokens = 0;       // one block per chunk after all
             if (int rc = launch_quantize_tables(kv, kv_dt, L, T, H, D, sl, skv, st, sh, key_bins, value_bins, sym4, maxima,
-                                                reinterpret_cast<uint16_t *>(cdf), w.nsub, chunk_tokens, nibbles, status, shape, s)) return rc;
+                                                reinterpret_cast<uint16_t *>(cdf), w.nsub, chunk_tokens, nibbles, status, shape, s,
+                                                nparts > 1 ? part_tokens : 0, nparts > 1 && part_tokens ? w.scratch : nullptr, slots_bytes)) return rc;
             return code_and_compact(o, sym4, nullptr, w, L, T, C, chunk_tokens, s, maxima, kv_dt, nibbles, true);
         }
         if (int rc = launch_quantize_pack(kv, kv_dt, L, T, H, D, sl, skv, st, sh, key_bins, value_bins, sym4,

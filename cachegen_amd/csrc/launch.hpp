@@ -244,6 +244,10 @@ int launch_quantize_pack(const void *kv, int kv_dt, int64_t L, int64_t T, int64_
 
 // The quantizer that also builds the tables (quantize_tables_kernel): which of its forms takes a tensor of `nunits` units of 8 channels and tables of `lp` entries,
 // if any.
+// Chunks of a call with fewer (row, chunk) pairs than kQuantTablesMinBlocks are cut into parts,
+// whole sub-chunks each, until the launch has about this many blocks.
+constexpr int64_t kQuantTablesPartBlocks = 1024;
+
 struct QuantTablesShape {
     int nu, lp;
     size_t lds;
@@ -281,7 +285,27 @@ int launch_quantize_tables_form(const QuantTablesArgs &a, dim3 grid, hipStream_t
             asked.fetch_or(1ull << dev, std::memory_order_relaxed);
         }
     }
+    if (!a.partial) {
+        quantize_tables_kernel<DT, HC, NU, LP><<<grid, dim3(QuantTablesBlock<NU>::kThreads), Layout::kBytes, stream>>>(a);
+        return check_launch("quantize_tables");
+    }
+    // chunks cut into parts: counters summed in memory, then one block per (chunk, row) for the tables
+    if (Layout::kBytes > 64 * 1024) {
+        static std::atomic<uint64_t> asked{0};
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return fail(CG_ERR_LAUNCH, "quantize_tables: hipGetDevice");
+        if (!(asked.load(std::memory_order_relaxed) >> dev & 1)) {
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&tables_from_partial_kernel<NU, LP>),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, Layout::kBytes);
+            if (e != hipSuccess) return fail(CG_ERR_LAUNCH, "quantize_tables: hipFuncSetAttribute: %s", hipGetErrorString(e));
+            asked.fetch_or(1ull << dev, std::memory_order_relaxed);
+        }
+    }
+    const int64_t nquads = (int64_t)grid.x * grid.y * (Layout::kBytes / 16);
+    clear_quads_kernel<<<dim3((unsigned)ceil_div(nquads, 256)), dim3(256), 0, stream>>>(reinterpret_cast<uint4 *>(a.partial), nquads);
     quantize_tables_kernel<DT, HC, NU, LP><<<grid, dim3(QuantTablesBlock<NU>::kThreads), Layout::kBytes, stream>>>(a);
+    tables_from_partial_kernel<NU, LP><<<dim3(grid.x, grid.y), dim3(QuantTablesBlock<NU>::kThreads), Layout::kBytes, stream>>>(
+        a.partial, a.cdf, a.nunits, a.g);
     return check_launch("quantize_tables");
 }
 
@@ -311,7 +335,8 @@ int launch_quantize_tables(const void *kv, int kv_dt, int64_t L, int64_t T, int6
                            int64_t sl, int64_t skv, int64_t st, int64_t sh, const float *key_bins,
                            const float *value_bins, uint32_t *sym4, void *maxima, uint16_t *cdf, int64_t nsub, int64_t S,
                            bool nibbles, int32_t *status,
-                           const QuantTablesShape &shape, hipStream_t stream)
+                           const QuantTablesShape &shape, hipStream_t stream,
+                           int64_t part_tokens = 0, void *partial = nullptr, size_t partial_bytes = 0)
 {
     QuantTablesArgs a;
     memset(&a, 0, sizeof(a));
@@ -336,7 +361,16 @@ int launch_quantize_tables(const void *kv, int kv_dt, int64_t L, int64_t T, int6
     a.g.nsc = (int32_t)ceil_div(S, kSub);
     const int64_t nchunks = ceil_div(T, S);
     if (nchunks > INT_MAX || 2 * L > 65535) return fail(CG_ERR_ARG, "quantize_tables: grid out of range");
-    const dim3 grid((unsigned)nchunks, (unsigned)(2 * L));
+    dim3 grid((unsigned)nchunks, (unsigned)(2 * L));
+    if (partial) {
+        const int64_t nparts = ceil_div(S < T ? S : T, part_tokens);
+        if (part_tokens <= 0 || part_tokens % kSub || nparts > 65535 || !aligned_to(partial, 16) ||
+            (size_t)nchunks * 2 * L * shape.lds > partial_bytes)
+            return fail(CG_ERR_ARG, "quantize_tables: parts of chunks out of range");
+        grid.z = (unsigned)nparts;
+        a.part_tokens = (int32_t)part_tokens;
+        a.partial = static_cast<uint32_t *>(partial);
+    }
     const bool contiguous = (sh == D);
     if (kv_dt == CG_DT_F16) {
         if (contiguous) return launch_quantize_tables_shape<CG_DT_F16, true>(a, shape, grid, stream);

@@ -44,6 +44,12 @@ struct QuantTablesArgs {
     int64_t nsub;
     int32_t nibbles;        // rows of at most 15 symbols are written four bits a symbol
     TokenGeom g;
+    // A call with few (row, chunk) pairs and long chunks cuts every chunk into gridDim.z parts of
+    // part_tokens tokens (a multiple of 256), one block each: a block then adds its counters to
+    // the chunk's words of `partial` (the layout of the LDS counters, zero before the launch)
+    // instead of writing tables, and tables_from_partial_kernel turns the sums into the tables.
+    int32_t part_tokens;
+    uint32_t *partial;      // null: one block per chunk, which writes the chunk's tables itself
 };
 
 // Lanes per block.  The counters of 1024 channels (33-entry tables) take 66 KiB, so two blocks
@@ -87,6 +93,75 @@ __device__ __forceinline__ uint32_t normalized_entry(uint32_t run, uint32_t entr
     return (q + entry) & 0xFFFFu;
 }
 
+// The tables of one (row, chunk) from its counters in LDS (every thread of the block, after a
+// barrier that follows the last count): `total` tokens were counted, `dst_tables` = the chunk's
+// [channel][LP] entries.
+template <int NU, int LP, int kThreads>
+__device__ __forceinline__ void counts_to_tables(uint32_t *counts, uint32_t total, int nunits, uint16_t *dst_tables)
+{
+    typedef CountLayout<NU, LP> Layout;
+    const int tid = threadIdx.x;
+    // One thread per channel pair (the two halves of a counter word).  The 2 LP counts are read
+    // in LP reads on immediate offsets; running sums and normalisation (cal_cdf.cu:11-14, 29-49)
+    // happen in registers; the pair's two tables, which follow one another in memory, go back to
+    // the LDS as LP words in the order of the output, from where the block writes its 2 * LP * C
+    // bytes of tables with coalesced 128-bit stores.
+    const bool shift = (total & (total - 1)) == 0;
+    const int sh = 31 - __builtin_clz(total);
+    const float inv = __fdiv_rn(1.0f, (float)total);
+    constexpr uint32_t scale = 0xFFFFu - (uint32_t)(LP - 1);
+    constexpr int kPairs = Layout::kSubTables * 64;
+    static_assert(kPairs % kThreads == 0 || kPairs < kThreads, "");
+    constexpr int kRounds = (kPairs + kThreads - 1) / kThreads;
+    uint32_t cnt[kRounds][LP];
+#pragma unroll
+    for (int r = 0; r < kRounds; ++r) {
+        const int p = tid + r * kThreads;
+        const int idx = p >> 6, ln = p & 63;
+        if (p < kPairs) {
+            const uint32_t *w = counts + (Layout::group_base(idx) + Layout::sub_table(idx)) / 4 + ln;
+#pragma unroll
+            for (int e = 0; e < LP; ++e) cnt[r][e] = w[e * 64];
+        }
+    }
+    __syncthreads();                         // every count is in registers: the LDS is free for the tables
+#pragma unroll
+    for (int r = 0; r < kRounds; ++r) {
+        const int p = tid + r * kThreads;
+        const int idx = p >> 6, ln = p & 63;
+        const int u = ln + 64 * (idx >> 2);
+        if (p < kPairs && u < nunits) {
+            // the pair's place in the output: channels 8 u + 2 kp and the next, LP words
+            uint32_t *dst = counts + ((int64_t)u * 4 + (idx & 3)) * LP;
+            auto emit = [&](auto shift_tag) {
+                constexpr bool SHIFT = decltype(shift_tag)::value;
+                uint32_t ra = 0, rb = 0, pa = 0, pb = 0, b0 = 0;
+#pragma unroll
+                for (int e = 0; e < LP; ++e) {
+                    ra += cnt[r][e] & 0xFFFFu;
+                    rb += cnt[r][e] >> 16;
+                    const uint32_t va = normalized_entry<SHIFT>(ra, (uint32_t)e, scale, total, sh, inv);
+                    const uint32_t vb = normalized_entry<SHIFT>(rb, (uint32_t)e, scale, total, sh, inv);
+                    // the sequence A[0..LP), B[0..LP) two entries a word
+                    if (e & 1) dst[e >> 1] = pa | (va << 16);                       // A[e-1], A[e]
+                    if (e == 0) b0 = vb;
+                    else if (!(e & 1)) dst[(LP + e - 1) >> 1] = pb | (vb << 16);    // B[e-1], B[e]
+                    if (e == LP - 1) dst[(LP - 1) >> 1] = va | (b0 << 16);          // A[LP-1], B[0]
+                    pa = va;
+                    pb = vb;
+                }
+            };
+            if (shift) emit(BoolTag<true>());
+            else emit(BoolTag<false>());
+        }
+    }
+    __syncthreads();
+    // C * LP 16-bit entries = C * LP / 8 quad words (C is a multiple of 8), 16-byte aligned in memory
+    uint4 *const tables = reinterpret_cast<uint4 *>(dst_tables);
+    const int nquads = nunits * LP;
+    for (int q = tid; q < nquads; q += kThreads) tables[q] = reinterpret_cast<const uint4 *>(counts)[q];
+}
+
 // LP: the table length, max_bins + 1 (odd).
 template <int DT, bool HEADS_CONTIGUOUS, int NU, int LP>
 __global__ __launch_bounds__(QuantTablesBlock<NU>::kThreads, 4) void quantize_tables_kernel(QuantTablesArgs a)
@@ -95,11 +170,22 @@ __global__ __launch_bounds__(QuantTablesBlock<NU>::kThreads, 4) void quantize_ta
     constexpr int kThreads = QuantTablesBlock<NU>::kThreads;
     extern __shared__ uint32_t counts[];
     typedef CountLayout<NU, LP> Layout;
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int tid = threadIdx.x, lane = tid & 63;
+    // the same for every lane of a wavefront, and said so: token rows, symbol and maxima
+    // addresses that depend on it are then computed once, on the scalar unit
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) *a.status = 0;
     const int64_t chunk = blockIdx.x, row = blockIdx.y;
-    const int64_t t0 = chunk * a.g.S;
-    const int ntok = (int)((t0 + a.g.S < a.g.T ? t0 + a.g.S : a.g.T) - t0);
+    // the block's tokens: the whole chunk, or part blockIdx.z of it (none, past the end of a short last chunk)
+    const int part_t0 = (int)blockIdx.z * a.part_tokens;         // 0 when chunks are not cut
+    const int64_t t0 = chunk * a.g.S + part_t0;
+    int ntok;
+    {
+        const int64_t chunk_end = (chunk + 1) * a.g.S < a.g.T ? (chunk + 1) * a.g.S : a.g.T;
+        const int64_t left = chunk_end - t0;
+        ntok = (int)(left < 0 ? 0 : a.partial && left > a.part_tokens ? a.part_tokens : left);
+    }
+    const int64_t sub0 = chunk * a.g.nsc + (part_t0 >> 8);       // the block's first sub-chunk
     const int64_t kvi = row / a.L, l = row - kvi * a.L;
     const float bins = (kvi ? a.value_bins : a.key_bins)[l];
     const float maxq = floorf(bins * 0.5f) - 1.0f;
@@ -156,7 +242,7 @@ __global__ __launch_bounds__(QuantTablesBlock<NU>::kThreads, 4) void quantize_ta
 
     // maxima, scales and counts of group tg, whose rows are in `regs`
     auto consume = [&](int tg, const uint4 (&regs)[4][NU]) {
-        const int tt0 = tg * 4;                              // first token of the group, inside the chunk
+        const int tt0 = tg * 4;                              // first token of the group, counted from the block's first
         const int nvalid = ntok - tt0 < 4 ? ntok - tt0 : 4;
         float factor[4];
         bool plain = fits;                                   // uniform over the wavefront
@@ -177,7 +263,7 @@ __global__ __launch_bounds__(QuantTablesBlock<NU>::kThreads, 4) void quantize_ta
             if (j < nvalid && lane == 0) a.maxima[row * a.g.T + t0 + tt0 + j] = (uint16_t)m;
             plain = plain && !scale_overflows(maxq, mf);
         }
-        const int64_t sub = chunk * a.g.nsc + (tt0 >> 8);
+        const int64_t sub = sub0 + (tt0 >> 8);
         uint32_t *out = a.sym4 + ((row * a.nsub + sub) * kWordsPerSub + ((tt0 & (kSub - 1)) >> 2)) * C;
 #pragma unroll
         for (int i = 0; i < NU; ++i) {
@@ -248,67 +334,44 @@ __global__ __launch_bounds__(QuantTablesBlock<NU>::kThreads, 4) void quantize_ta
         }
     }
 
-    // One thread per channel pair (the two halves of a counter word).  The 2 LP counts are read
-    // in LP reads on immediate offsets; running sums and normalisation (cal_cdf.cu:11-14, 29-49)
-    // happen in registers; the pair's two tables, which follow one another in memory, go back to
-    // the LDS as LP words in the order of the output, from where the block writes its 2 * LP * C
-    // bytes of tables with coalesced 128-bit stores.
     __syncthreads();
-    const uint32_t total = (uint32_t)ntok;
-    const bool shift = (total & (total - 1)) == 0;
-    const int sh = 31 - __builtin_clz(total);
-    const float inv = __fdiv_rn(1.0f, (float)total);
-    constexpr uint32_t scale = 0xFFFFu - (uint32_t)(LP - 1);
-    constexpr int kPairs = Layout::kSubTables * 64;
-    static_assert(kPairs % kThreads == 0 || kPairs < kThreads, "");
-    constexpr int kRounds = (kPairs + kThreads - 1) / kThreads;
-    uint32_t cnt[kRounds][LP];
-#pragma unroll
-    for (int r = 0; r < kRounds; ++r) {
-        const int p = tid + r * kThreads;
-        const int idx = p >> 6, ln = p & 63;
-        if (p < kPairs) {
-            const uint32_t *w = counts + (Layout::group_base(idx) + Layout::sub_table(idx)) / 4 + ln;
-#pragma unroll
-            for (int e = 0; e < LP; ++e) cnt[r][e] = w[e * 64];
+    if (a.partial) {
+        // the chunk's other parts add to the same words; what a block has not counted it does not touch
+        uint32_t *sums = a.partial + ((int64_t)blockIdx.x * gridDim.y + blockIdx.y) * (Layout::kBytes / 4);
+        for (int i = tid; i < Layout::kBytes / 4; i += kThreads) {
+            const uint32_t v = counts[i];
+            if (v) __hip_atomic_fetch_add(sums + i, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
+        return;
     }
-    __syncthreads();                         // every count is in registers: the LDS is free for the tables
-#pragma unroll
-    for (int r = 0; r < kRounds; ++r) {
-        const int p = tid + r * kThreads;
-        const int idx = p >> 6, ln = p & 63;
-        const int u = ln + 64 * (idx >> 2);
-        if (p < kPairs && u < a.nunits) {
-            // the pair's place in the output: channels 8 u + 2 kp and the next, LP words
-            uint32_t *dst = counts + ((int64_t)u * 4 + (idx & 3)) * LP;
-            auto emit = [&](auto shift_tag) {
-                constexpr bool SHIFT = decltype(shift_tag)::value;
-                uint32_t ra = 0, rb = 0, pa = 0, pb = 0, b0 = 0;
-#pragma unroll
-                for (int e = 0; e < LP; ++e) {
-                    ra += cnt[r][e] & 0xFFFFu;
-                    rb += cnt[r][e] >> 16;
-                    const uint32_t va = normalized_entry<SHIFT>(ra, (uint32_t)e, scale, total, sh, inv);
-                    const uint32_t vb = normalized_entry<SHIFT>(rb, (uint32_t)e, scale, total, sh, inv);
-                    // the sequence A[0..LP), B[0..LP) two entries a word
-                    if (e & 1) dst[e >> 1] = pa | (va << 16);                       // A[e-1], A[e]
-                    if (e == 0) b0 = vb;
-                    else if (!(e & 1)) dst[(LP + e - 1) >> 1] = pb | (vb << 16);    // B[e-1], B[e]
-                    if (e == LP - 1) dst[(LP - 1) >> 1] = va | (b0 << 16);          // A[LP-1], B[0]
-                    pa = va;
-                    pb = vb;
-                }
-            };
-            if (shift) emit(BoolTag<true>());
-            else emit(BoolTag<false>());
-        }
-    }
+    counts_to_tables<NU, LP, kThreads>(counts, (uint32_t)ntok, a.nunits,
+                                       a.cdf + (((int64_t)blockIdx.x * gridDim.y + blockIdx.y) * a.nunits * 8) * LP);
+}
+
+// Zeroes n quad words (the counters in memory, before the blocks of a launch add to them).
+__global__ __launch_bounds__(256) void clear_quads_kernel(uint4 *p, int64_t n)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) p[i] = make_uint4(0, 0, 0, 0);
+}
+
+// The tables of the chunks whose counters quantize_tables_kernel summed in memory: a block per
+// (chunk, row) copies the sums into its LDS and goes on as that kernel does at the end of a chunk.
+template <int NU, int LP>
+__global__ __launch_bounds__(QuantTablesBlock<NU>::kThreads, 4) void tables_from_partial_kernel(
+    const uint32_t *__restrict__ partial, uint16_t *cdf, int32_t nunits, TokenGeom g)
+{
+    constexpr int kThreads = QuantTablesBlock<NU>::kThreads;
+    extern __shared__ uint32_t counts[];
+    typedef CountLayout<NU, LP> Layout;
+    const int tid = threadIdx.x;
+    const int64_t chunk = blockIdx.x, row = blockIdx.y;
+    const int64_t t0 = chunk * g.S;
+    const uint32_t total = (uint32_t)((t0 + g.S < g.T ? t0 + g.S : g.T) - t0);
+    const uint4 *src = reinterpret_cast<const uint4 *>(partial + (chunk * gridDim.y + row) * (Layout::kBytes / 4));
+    for (int i = tid; i < Layout::kBytes / 16; i += kThreads) reinterpret_cast<uint4 *>(counts)[i] = src[i];
     __syncthreads();
-    // C * LP 16-bit entries = C * LP / 8 quad words (C is a multiple of 8), 16-byte aligned in memory
-    uint4 *const tables = reinterpret_cast<uint4 *>(a.cdf + ((chunk * gridDim.y + row) * C) * LP);
-    const int nquads = (int)(C * LP / 8);
-    for (int q = tid; q < nquads; q += kThreads) tables[q] = reinterpret_cast<const uint4 *>(counts)[q];
+    counts_to_tables<NU, LP, kThreads>(counts, total, nunits, cdf + ((chunk * gridDim.y + row) * (int64_t)nunits * 8) * LP);
 }
 
 }  // namespace

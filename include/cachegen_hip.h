@@ -162,12 +162,16 @@ int cg_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int
  *                               symbol (cg_encode_kv packs rows of at most 15 symbols four bits a symbol)
  * CG_TEST_TABLES_IN_QUANTIZER   the quantizer counts the symbols and writes the tables, however few
  *                               chunks the call has (cg_encode_kv does so from 512 (row, chunk) pairs on,
- *                               where the tables of all channels fit the LDS of one block)
+ *                               where the tables of all channels fit the LDS of one block; calls with
+ *                               fewer pairs and chunks of more than 256 tokens cut the chunks into parts)
+ * CG_TEST_SPLIT_CHUNKS          with the form above: every chunk of more than 256 tokens is counted in
+ *                               parts of 256 tokens by separate blocks, whose counters are summed in memory
  * CG_TEST_TABLES_IN_CODER       never: the coder (one table per sub-chunk) or a separate pass over
  *                               the symbols (longer chunks) builds the tables */
 #define CG_TEST_BYTE_SYMBOLS 1
 #define CG_TEST_TABLES_IN_QUANTIZER 2
 #define CG_TEST_TABLES_IN_CODER 4
+#define CG_TEST_SPLIT_CHUNKS 8
 int cg_test_encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_t D,
                       int64_t sl, int64_t skv, int64_t st, int64_t sh,
                       const float *key_bins, const float *value_bins, int max_bins,

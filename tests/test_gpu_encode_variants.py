@@ -6,6 +6,9 @@ encoder.py:42-59, and calculate_cdf, cal_cdf.cu:17-59, in one pass) when the cal
 chunk) pairs enough to fill the GPU, else the coder or a separate pass over the symbols does.
 The small inputs the oracle can follow would never take the first form by themselves, so the
 library's test entry point forces each form here; every form is compared with the oracle.
+A call with few (row, chunk) pairs but long chunks (the reference serializer's one table over a
+whole context) cuts each chunk into parts counted by separate blocks, whose counters are summed in
+memory before the tables are made: SPLIT_CHUNKS forces parts of 256 tokens.
 """
 import numpy as np
 import pytest
@@ -14,7 +17,7 @@ import torch
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
-BYTE_SYMBOLS, TABLES_IN_QUANTIZER, TABLES_IN_CODER = 1, 2, 4
+BYTE_SYMBOLS, TABLES_IN_QUANTIZER, TABLES_IN_CODER, SPLIT_CHUNKS = 1, 2, 4, 8
 
 
 def bits(t):
@@ -69,11 +72,12 @@ def test_every_form_of_the_encoder_matches_the_oracle(oracle, dtype, dt, L, T, H
     plain = codec.encode_kv(dev, kb, vb, chunk_tokens=S)
     plain.check()
     _against_oracle(oracle, plain, kv, kb, vb, S, dt)
-    for flags in (TABLES_IN_QUANTIZER, TABLES_IN_CODER, TABLES_IN_QUANTIZER | BYTE_SYMBOLS, TABLES_IN_CODER | BYTE_SYMBOLS):
+    for flags in (TABLES_IN_QUANTIZER, TABLES_IN_CODER, TABLES_IN_QUANTIZER | BYTE_SYMBOLS, TABLES_IN_CODER | BYTE_SYMBOLS,
+                  TABLES_IN_QUANTIZER | SPLIT_CHUNKS, TABLES_IN_QUANTIZER | SPLIT_CHUNKS | BYTE_SYMBOLS):
         other = codec.encode_kv(dev, kb, vb, chunk_tokens=S, _test_flags=flags)
         other.check()
         _same(plain, other)
-        if flags == TABLES_IN_QUANTIZER:
+        if flags in (TABLES_IN_QUANTIZER, TABLES_IN_QUANTIZER | SPLIT_CHUNKS):
             _against_oracle(oracle, other, kv, kb, vb, S, dt)
 
 
@@ -96,7 +100,7 @@ def test_forms_agree_on_the_other_layout_and_on_saturated_rows(oracle):
     for fmt, dev in (("vllm", kv.to(DEV)), ("huggingface", hf)):
         for max_bins in (None, 12):
             base = codec.encode_kv(dev, kb, vb, chunk_tokens=260, fmt=fmt, max_bins=max_bins, _test_flags=TABLES_IN_CODER)
-            for flags in (TABLES_IN_QUANTIZER, TABLES_IN_QUANTIZER | BYTE_SYMBOLS):
+            for flags in (TABLES_IN_QUANTIZER, TABLES_IN_QUANTIZER | BYTE_SYMBOLS, TABLES_IN_QUANTIZER | SPLIT_CHUNKS):
                 _same(base, codec.encode_kv(dev, kb, vb, chunk_tokens=260, fmt=fmt, max_bins=max_bins, _test_flags=flags))
 
 
@@ -116,5 +120,16 @@ def test_default_call_takes_the_quantizer_form_at_benchmark_size():
     # chunks of 1500 tokens: six sub-chunks under one table
     a = codec.encode_kv(kv, kb, vb, chunk_tokens=1500)
     b = codec.encode_kv(kv, kb, vb, chunk_tokens=1500, _test_flags=TABLES_IN_CODER)
+    a.check()
+    _same(a, b)
+    # one table over the whole context, the reference serializer's own call: 64 (row, chunk) pairs,
+    # so every chunk is counted in parts of 512 tokens
+    a = codec.encode_kv(kv, kb, vb, chunk_tokens=8192)
+    b = codec.encode_kv(kv, kb, vb, chunk_tokens=8192, _test_flags=TABLES_IN_CODER)
+    a.check()
+    _same(a, b)
+    # three chunks of 3000 tokens (the last one 2192): parts of 256 tokens
+    a = codec.encode_kv(kv, kb, vb, chunk_tokens=3000)
+    b = codec.encode_kv(kv, kb, vb, chunk_tokens=3000, _test_flags=TABLES_IN_CODER)
     a.check()
     _same(a, b)

@@ -64,6 +64,13 @@ def test_random_wide_case_with_tables_built_by_the_quantizer(oracle, seed):
     run_cases(oracle, seed, 2, True, flags=2)
 
 
+@pytest.mark.parametrize("seed", range(24, 32))
+def test_random_case_with_chunks_counted_in_parts(oracle, seed):
+    """The quantizer-built tables with every chunk of more than 256 tokens cut into parts of 256
+    tokens that separate blocks count (CG_TEST_SPLIT_CHUNKS), as calls with few long chunks do."""
+    run_cases(oracle, seed, 4, False, flags=2 | 8)
+
+
 def run_cases(oracle, seed, ncases, wide, flags=None):
     from cachegen_amd import codec
     from cachegen_amd.kvgen import make_kv

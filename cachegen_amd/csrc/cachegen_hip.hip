@@ -436,7 +436,7 @@ int encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_
         // (in the stream slots of the workspace, which nothing uses before the coder runs).
         int64_t part_tokens = 0;
         if ((flags & CG_TEST_SPLIT_CHUNKS) && reach > kSub) part_tokens = kSub;
-        else if (2 * L * nchunks < kQuantTablesMinBlocks && reach > kSub) {
+        else if (2 * L * nchunks < kQuantTablesPartBlocks && reach > kSub) {
             const int64_t want = ceil_div(kQuantTablesPartBlocks, 2 * L * nchunks);     // parts per chunk
             part_tokens = reach / want / kSub * kSub;
             if (part_tokens < kSub) part_tokens = kSub;

@@ -244,9 +244,10 @@ int launch_quantize_pack(const void *kv, int kv_dt, int64_t L, int64_t T, int64_
 
 // The quantizer that also builds the tables (quantize_tables_kernel): which of its forms takes a tensor of `nunits` units of 8 channels and tables of `lp` entries,
 // if any.
-// Chunks of a call with fewer (row, chunk) pairs than kQuantTablesMinBlocks are cut into parts,
-// whole sub-chunks each, until the launch has about this many blocks.
-constexpr int64_t kQuantTablesPartBlocks = 1024;
+// Long chunks of a call with fewer (row, chunk) pairs than this are cut into parts, whole
+// sub-chunks each, until the launch has about this many blocks (measured on one table over
+// 8192 tokens of 32 layers: parts of 256 tokens 0.765 ms, of 512 tokens 0.807, the whole encode).
+constexpr int64_t kQuantTablesPartBlocks = 2048;
 
 struct QuantTablesShape {
     int nu, lp;
@@ -268,39 +269,33 @@ bool quantize_tables_shape(int64_t nunits, int lp, bool heads_contiguous, QuantT
     return shape.lds <= kMaxLdsPerBlock;
 }
 
+// A kernel that wants more than 64 KiB of dynamic LDS has to be allowed to, once per device;
+// `asked` holds one bit per device for that kernel.
+int allow_dynamic_lds(const void *kernel, int bytes, std::atomic<uint64_t> &asked)
+{
+    if (bytes <= 64 * 1024) return CG_OK;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return fail(CG_ERR_LAUNCH, "quantize_tables: hipGetDevice");
+    if (asked.load(std::memory_order_relaxed) >> dev & 1) return CG_OK;
+    const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess) return fail(CG_ERR_LAUNCH, "quantize_tables: hipFuncSetAttribute: %s", hipGetErrorString(e));
+    asked.fetch_or(1ull << dev, std::memory_order_relaxed);
+    return CG_OK;
+}
+
 template <int DT, bool HC, int NU, int LP>
 int launch_quantize_tables_form(const QuantTablesArgs &a, dim3 grid, hipStream_t stream)
 {
     typedef CountLayout<NU, LP> Layout;
     if (Layout::kBytes > (int)kMaxLdsPerBlock) return fail(CG_ERR_ARG, "quantize_tables: tables do not fit the LDS");
-    if (Layout::kBytes > 64 * 1024) {
-        // more than 64 KiB of dynamic LDS has to be asked for, once per device
-        static std::atomic<uint64_t> asked{0};
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return fail(CG_ERR_LAUNCH, "quantize_tables: hipGetDevice");
-        if (!(asked.load(std::memory_order_relaxed) >> dev & 1)) {
-            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&quantize_tables_kernel<DT, HC, NU, LP>),
-                                                     hipFuncAttributeMaxDynamicSharedMemorySize, Layout::kBytes);
-            if (e != hipSuccess) return fail(CG_ERR_LAUNCH, "quantize_tables: hipFuncSetAttribute: %s", hipGetErrorString(e));
-            asked.fetch_or(1ull << dev, std::memory_order_relaxed);
-        }
-    }
+    static std::atomic<uint64_t> asked{0}, asked_for_sums{0};       // per form of the kernel: these are templates
+    if (int rc = allow_dynamic_lds(reinterpret_cast<const void *>(&quantize_tables_kernel<DT, HC, NU, LP>), Layout::kBytes, asked)) return rc;
     if (!a.partial) {
         quantize_tables_kernel<DT, HC, NU, LP><<<grid, dim3(QuantTablesBlock<NU>::kThreads), Layout::kBytes, stream>>>(a);
         return check_launch("quantize_tables");
     }
     // chunks cut into parts: counters summed in memory, then one block per (chunk, row) for the tables
-    if (Layout::kBytes > 64 * 1024) {
-        static std::atomic<uint64_t> asked{0};
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return fail(CG_ERR_LAUNCH, "quantize_tables: hipGetDevice");
-        if (!(asked.load(std::memory_order_relaxed) >> dev & 1)) {
-            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&tables_from_partial_kernel<NU, LP>),
-                                                     hipFuncAttributeMaxDynamicSharedMemorySize, Layout::kBytes);
-            if (e != hipSuccess) return fail(CG_ERR_LAUNCH, "quantize_tables: hipFuncSetAttribute: %s", hipGetErrorString(e));
-            asked.fetch_or(1ull << dev, std::memory_order_relaxed);
-        }
-    }
+    if (int rc = allow_dynamic_lds(reinterpret_cast<const void *>(&tables_from_partial_kernel<NU, LP>), Layout::kBytes, asked_for_sums)) return rc;
     const int64_t nquads = (int64_t)grid.x * grid.y * (Layout::kBytes / 16);
     clear_quads_kernel<<<dim3((unsigned)ceil_div(nquads, 256)), dim3(256), 0, stream>>>(reinterpret_cast<uint4 *>(a.partial), nquads);
     quantize_tables_kernel<DT, HC, NU, LP><<<grid, dim3(QuantTablesBlock<NU>::kThreads), Layout::kBytes, stream>>>(a);

@@ -123,13 +123,15 @@ def test_default_call_takes_the_quantizer_form_at_benchmark_size():
     a.check()
     _same(a, b)
     # one table over the whole context, the reference serializer's own call: 64 (row, chunk) pairs,
-    # so every chunk is counted in parts of 512 tokens
+    # so every chunk is counted in parts of 256 tokens
     a = codec.encode_kv(kv, kb, vb, chunk_tokens=8192)
     b = codec.encode_kv(kv, kb, vb, chunk_tokens=8192, _test_flags=TABLES_IN_CODER)
     a.check()
     _same(a, b)
-    # three chunks of 3000 tokens (the last one 2192): parts of 256 tokens
-    a = codec.encode_kv(kv, kb, vb, chunk_tokens=3000)
-    b = codec.encode_kv(kv, kb, vb, chunk_tokens=3000, _test_flags=TABLES_IN_CODER)
-    a.check()
-    _same(a, b)
+    # three chunks of 3000 tokens (the last one 2192, so some parts hold no token); and chunks of
+    # 1024 tokens: 512 pairs, cut as well
+    for S in (3000, 1024):
+        a = codec.encode_kv(kv, kb, vb, chunk_tokens=S)
+        b = codec.encode_kv(kv, kb, vb, chunk_tokens=S, _test_flags=TABLES_IN_CODER)
+        a.check()
+        _same(a, b)

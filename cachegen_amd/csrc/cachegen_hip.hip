@@ -248,7 +248,7 @@ struct EncodeWorkspace {
     size_t symbols_bytes;       // one level's symbols
     uint8_t *symbols, *scratch;
     void *scan_scratch, *tile_scan_scratch;
-    int32_t *tile_sums;
+    int32_t *tile_sums, *group_sums;
     int64_t *tile_base;
     int64_t nsub, nstreams, ntiles;
     size_t total;
@@ -272,6 +272,8 @@ struct EncodeWorkspace {
         ws += align_up((size_t)(ntiles + 1) * sizeof(int64_t), 256);
         tile_scan_scratch = ws;
         ws += cg_scan_workspace(ntiles);
+        group_sums = reinterpret_cast<int32_t *>(ws);          // bytes per group of kTileGroup tiles
+        ws += align_up((size_t)kMaxTileGroups * sizeof(int32_t), 256);
         total = (size_t)(ws - static_cast<uint8_t *>(base));
     }
 };
@@ -313,7 +315,8 @@ struct LevelOut {
 // The level's status word has been set to zero by an earlier launch of the same call.
 // maxima, max_dt: the row maxima (packed symbols only); nibbles: the quantizer packed the rows
 // of at most 15 symbols four bits a symbol (see narrow_alphabet).
-// tables_ready: the tables were written by an earlier launch of the call (quantize_tables_kernel).
+// tables_ready: the tables were written by an earlier launch of the call (quantize_tables_kernel),
+// which also set the workspace's group sums to zero.
 int code_and_compact(const LevelOut &o, const uint32_t *sym4, const uint8_t *sym_bytes, const EncodeWorkspace &w,
                      int64_t L, int64_t T, int64_t C, int64_t chunk_tokens, hipStream_t s,
                      const void *maxima = nullptr, int max_dt = 0, bool nibbles = false, bool tables_ready = false)
@@ -343,6 +346,11 @@ int code_and_compact(const LevelOut &o, const uint32_t *sym4, const uint8_t *sym
     // counts behind and the compaction computes the stream offsets itself
     const bool fused_scan = block == kSlotTile && C % kSlotTile == 0;
     a.tile_sums = fused_scan ? w.tile_sums : nullptr;
+    // few enough tiles: no scan launch either, the coder's blocks add the counts up by groups of
+    // tiles (the sums were cleared by the quantizer that made the tables) and the compaction adds
+    // up what lies before each tile
+    const bool grouped = fused_scan && tables_ready && ceil_div(w.ntiles, kTileGroup) <= kMaxTileGroups;
+    a.group_sums = grouped ? w.group_sums : nullptr;
 
     if (sym4) {
         // four tokens per word, read by one lane per channel
@@ -377,7 +385,11 @@ int code_and_compact(const LevelOut &o, const uint32_t *sym4, const uint8_t *sym
     const int64_t cblocks = ceil_div(w.nstreams, kCompactStreams);
     if (cblocks > INT_MAX) return fail(CG_ERR_ARG, "encode_kv: too many streams");
     const int32_t skew = (int32_t)(reinterpret_cast<uintptr_t>(o.payload) & 3u);
-    if (fused_scan) {
+    if (grouped) {
+        compact_streams_kernel<true><<<dim3((unsigned)cblocks), dim3(256), 0, s>>>(
+            w.scratch, kStreamCap, o.offsets, o.lengths, nullptr, w.nstreams, o.payload, o.payload_cap, skew, o.status,
+            w.group_sums, w.tile_sums);
+    } else if (fused_scan) {
         if (int rc = launch_scan(w.tile_sums, cblocks, INT_MAX, w.tile_base, w.tile_scan_scratch, s)) return rc;
         compact_streams_kernel<true><<<dim3((unsigned)cblocks), dim3(256), 0, s>>>(
             w.scratch, kStreamCap, o.offsets, o.lengths, w.tile_base, w.nstreams, o.payload, o.payload_cap, skew, o.status);
@@ -451,7 +463,8 @@ int encode_kv(const void *kv, int kv_dt, int64_t L, int64_t T, int64_t H, int64_
             if (nparts > 1 && (size_t)nchunks * 2 * L * shape.lds > slots_bytes) part_tokens = 0;       // one block per chunk after all
             if (int rc = launch_quantize_tables(kv, kv_dt, L, T, H, D, sl, skv, st, sh, key_bins, value_bins, sym4, maxima,
                                                 reinterpret_cast<uint16_t *>(cdf), w.nsub, chunk_tokens, nibbles, status, shape, s,
-                                                nparts > 1 ? part_tokens : 0, nparts > 1 && part_tokens ? w.scratch : nullptr, slots_bytes)) return rc;
+                                                nparts > 1 ? part_tokens : 0, nparts > 1 && part_tokens ? w.scratch : nullptr, slots_bytes,
+                                                w.group_sums)) return rc;
             return code_and_compact(o, sym4, nullptr, w, L, T, C, chunk_tokens, s, maxima, kv_dt, nibbles, true);
         }
         if (int rc = launch_quantize_pack(kv, kv_dt, L, T, H, D, sl, skv, st, sh, key_bins, value_bins, sym4,

@@ -30,6 +30,11 @@ namespace {
 // whether the carry comes.  n <= 18 for any table whose symbols all have non-zero width,
 // because the span stays above 2^30 between symbols.
 constexpr int kSlotTile = 256;      // streams per tile of the encoder's scratch
+// Tiles whose byte counts the coder's blocks also add up into one sum per group, so that the
+// compaction finds a tile's place in the payload from at most kMaxTileGroups group sums and
+// kTileGroup - 1 tile counts; calls with more groups run a scan launch over the tile counts.
+constexpr int kTileGroup = 64;
+constexpr int kMaxTileGroups = 256;
 
 // TILE: the stream's words go to a tile of the scratch (word w of the tile's stream t at the
 // tile's word w * kSlotTile + t) through a buffer descriptor that covers exactly the tile: a
@@ -313,6 +318,8 @@ struct EncodeArgs {
     int32_t *lengths;       // [sub][row][channel]
     int32_t *status;        // may be null
     int32_t *tile_sums;     // SLOTS, one block per tile of kSlotTile streams: stored bytes per tile, or null
+    int32_t *group_sums;    // with tile_sums, or null: the tile's bytes are also added to the sum of its
+                            // group of kTileGroup tiles (zero before the launch)
     const float *key_bins, *value_bins;     // float32 [L] each, or null when the levels are not known
     int64_t L;
     StreamGrid sg;
@@ -548,7 +555,9 @@ __global__ __launch_bounds__(BS) void encode_streams_kernel(EncodeArgs a)
         if (tid == 0) {
             int32_t total = 0;
             for (int w = 0; w < BS / 64; ++w) total += wave_sums[w];
-            a.tile_sums[linear_block()] = total;                  // at most 256 streams of 256 bytes
+            const uint32_t tile = linear_block();
+            a.tile_sums[tile] = total;                            // at most 256 streams of 256 bytes
+            if (a.group_sums) __hip_atomic_fetch_add(a.group_sums + tile / kTileGroup, total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
 }

@@ -331,7 +331,8 @@ int launch_quantize_tables(const void *kv, int kv_dt, int64_t L, int64_t T, int6
                            const float *value_bins, uint32_t *sym4, void *maxima, uint16_t *cdf, int64_t nsub, int64_t S,
                            bool nibbles, int32_t *status,
                            const QuantTablesShape &shape, hipStream_t stream,
-                           int64_t part_tokens = 0, void *partial = nullptr, size_t partial_bytes = 0)
+                           int64_t part_tokens = 0, void *partial = nullptr, size_t partial_bytes = 0,
+                           int32_t *group_sums = nullptr)
 {
     QuantTablesArgs a;
     memset(&a, 0, sizeof(a));
@@ -345,6 +346,8 @@ int launch_quantize_tables(const void *kv, int kv_dt, int64_t L, int64_t T, int6
     a.key_bins = key_bins;
     a.value_bins = value_bins;
     a.status = status;
+    a.group_sums = group_sums;          // kMaxTileGroups words of the workspace
+    a.ngroups = kMaxTileGroups;
     a.sym4 = sym4;
     a.maxima = static_cast<uint16_t *>(maxima);
     a.cdf = cdf;

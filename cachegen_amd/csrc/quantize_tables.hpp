@@ -37,6 +37,8 @@ struct QuantTablesArgs {
     int32_t D;
     const float *key_bins, *value_bins;
     int32_t *status;        // the encode call's status word, set to zero here (first launch of the call)
+    int32_t *group_sums;    // ngroups sums the coder's blocks add to, set to zero here (may be null)
+    int32_t ngroups;
     uint32_t *sym4;         // packed symbols, as quantize_pack_kernel writes them
     uint16_t *maxima;       // [2L, T]
     uint16_t *cdf;          // [chunk][row][channel][lp]
@@ -174,7 +176,10 @@ __global__ __launch_bounds__(QuantTablesBlock<NU>::kThreads, 4) void quantize_ta
     // the same for every lane of a wavefront, and said so: token rows, symbol and maxima
     // addresses that depend on it are then computed once, on the scalar unit
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) *a.status = 0;
+    if (blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0) {
+        if (tid == 0) *a.status = 0;
+        if (a.group_sums && tid < a.ngroups) a.group_sums[tid] = 0;          // ngroups <= kMaxTileGroups < the block's threads
+    }
     const int64_t chunk = blockIdx.x, row = blockIdx.y;
     // the block's tokens: the whole chunk, or part blockIdx.z of it (none, past the end of a short last chunk)
     const int part_t0 = (int)blockIdx.z * a.part_tokens;         // 0 when chunks are not cut

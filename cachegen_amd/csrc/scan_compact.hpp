@@ -193,12 +193,16 @@ constexpr int kCompactStreams = 256;
 constexpr int kCompactTile = 16384;
 
 // SCAN: the offsets are not known yet; `offsets` is written here from the streams' lengths and
-// the exclusive running sum of the tiles' byte counts (tile_base), instead of being read.
+// the exclusive running sum of the tiles' byte counts, instead of being read.  That sum comes
+// from tile_base (a scan launch made it), or, group_sums != null, is added up here: the sums of
+// the groups of kTileGroup tiles before this block's group (at most kMaxTileGroups, left by the
+// coder) and the counts of the tiles before this one in its group.
 template <bool SCAN>
 __global__ __launch_bounds__(256) void compact_streams_kernel(
     const uint8_t *__restrict__ slots, int32_t cap, int64_t *__restrict__ offsets,
     const int32_t *__restrict__ lengths, const int64_t *__restrict__ tile_base,
-    int64_t nstreams, uint8_t *__restrict__ payload, int64_t payload_cap, int32_t skew, int32_t *status)
+    int64_t nstreams, uint8_t *__restrict__ payload, int64_t payload_cap, int32_t skew, int32_t *status,
+    const int32_t *__restrict__ group_sums = nullptr, const int32_t *__restrict__ tile_sums = nullptr)
 {
     __shared__ int32_t rel[kCompactStreams + 1];       // stream offsets relative to the block's first byte
     __shared__ __align__(16) uint32_t buf[kCompactTile / 4];
@@ -212,8 +216,17 @@ __global__ __launch_bounds__(256) void compact_streams_kernel(
             mine = lengths[sbase + tid];
             mine = mine < 0 ? 0 : (mine > cap ? cap : mine);
         }
-        o0 = tile_base[blockIdx.x];
         int32_t total32;
+        if (group_sums) {
+            const int g = (int)(blockIdx.x / kTileGroup), r = (int)(blockIdx.x % kTileGroup);
+            int32_t part = tid < g ? group_sums[tid] : 0;
+            if (tid < r) part += tile_sums[(int64_t)g * kTileGroup + tid];
+            int32_t sum;
+            block_exclusive_scan_256(part, reinterpret_cast<int32_t *>(buf), sum);     // at most 16384 tiles of 64 KiB: fits
+            o0 = sum;
+        } else {
+            o0 = tile_base[blockIdx.x];
+        }
         const int32_t before = block_exclusive_scan_256(mine, reinterpret_cast<int32_t *>(buf), total32);    // buf is free until the copy
         const int64_t total64 = total32;                       // at most 256 streams of `cap` <= 256 bytes
         rel[tid] = before;

@@ -40,6 +40,11 @@ OCCUPANCY_BUDGETS = [
 ]
 
 
+# Kernels that address their dynamically allocated LDS from byte 0 (the counters of the table
+# builder: the address comes out of a byte permute): a statically allocated array would sit there.
+NO_STATIC_LDS = r"^(quantize_tables_kernel|tables_from_partial_kernel)<"
+
+
 def parse_kernel_resources(report):
     """{demangled kernel name: {"vgprs", "agprs", "sgprs", "scratch", "occupancy", "lds"}} from the
     remarks of -Rpass-analysis=kernel-resource-usage."""
@@ -74,6 +79,8 @@ def check_budgets(resources):
     for name, r in sorted(resources.items()):
         if r.get("scratch", 0) != 0:
             bad.append("%s spills %d bytes per lane to scratch memory" % (name, r["scratch"]))
+        if re.search(NO_STATIC_LDS, name) and r.get("lds", 0) != 0:
+            bad.append("%s has %d bytes of statically allocated LDS: its counters are addressed from LDS byte 0" % (name, r["lds"]))
         need = max([n for pat, n in OCCUPANCY_BUDGETS if re.search(pat, name)] or [0])
         if r.get("occupancy", 0) < need:
             bad.append("%s: %d wavefronts per SIMD (%d vector registers), budget %d"

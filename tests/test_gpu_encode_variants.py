@@ -135,3 +135,25 @@ def test_default_call_takes_the_quantizer_form_at_benchmark_size():
         b = codec.encode_kv(kv, kb, vb, chunk_tokens=S, _test_flags=TABLES_IN_CODER)
         a.check()
         _same(a, b)
+
+
+def test_largest_call_whose_tile_counts_are_summed_by_groups():
+    """16 384 scratch tiles (4 194 304 streams) is the most for which the compaction adds up group
+    sums and tile counts itself (256 groups of 64 tiles); one sub-chunk more and a scan launch
+    makes the running sum.  Both sides of the line against the form with the tables built in the
+    coder, which always runs the scan: same offsets, lengths and payload."""
+    from cachegen_amd import codec
+    from cachegen_amd.kvgen import make_kv
+    from cachegen_amd.serde import cachegen_basics as B
+    cfg = B.CacheGenConfig.from_model_name("lmsys/longchat-7b-16k")
+    kb, vb = B.make_key_bins(cfg).to(DEV), B.make_value_bins(cfg).to(DEV)
+    kv = make_kv(32, 16384 + 256, 8, 128, seed=77, device=DEV)
+    for T in (16384, 16384 + 256):
+        x = kv[:, :, :T]
+        a = codec.encode_kv(x, kb, vb, chunk_tokens=256)
+        b = codec.encode_kv(x, kb, vb, chunk_tokens=256, _test_flags=TABLES_IN_CODER)
+        a.check()
+        _same(a, b)
+        assert int(a.offsets[-1]) == a.total_bytes() == int(a.lengths.sum())
+        del a, b
+

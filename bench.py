@@ -155,7 +155,14 @@ def measured_counters():
         return json.load(f)
 
 
-def run_workload(name, steps, warmup, fmt="vllm", copy_probe=False, keep=False, ramp_ms=0.0, sample_clock=False):
+# --encode-form: the library's internal forms of the encode call, forced through its test entry
+# point (cg_test_encode_kv); the results are the same bytes, the profiles compare their cost
+ENCODE_FORMS = {"default": None, "tables-in-quantizer": 2, "tables-in-coder": 4, "byte-symbols": 1,
+                "tables-in-coder+byte-symbols": 5, "chunks-in-parts": 2 | 8}
+
+
+def run_workload(name, steps, warmup, fmt="vllm", copy_probe=False, keep=False, ramp_ms=0.0, sample_clock=False,
+                 encode_form="default"):
     """Encode + decode of one workload, timed with HIP events on the launching stream.
     Returns a dict of figures (and, with keep=True, the tensors for further use)."""
     import torch
@@ -173,7 +180,8 @@ def run_workload(name, steps, warmup, fmt="vllm", copy_probe=False, keep=False, 
     max_bins = int(max(kbins.max(), vbins.max()))
 
     workspace = torch.empty(codec.encode_workspace_bytes(L, T, C, chunk), dtype=torch.uint8, device=dev)
-    enc = codec.encode_kv(kv, kb, vb, chunk_tokens=chunk, max_bins=max_bins, workspace=workspace, fmt=fmt)
+    flags = ENCODE_FORMS[encode_form]
+    enc = codec.encode_kv(kv, kb, vb, chunk_tokens=chunk, max_bins=max_bins, workspace=workspace, fmt=fmt, _test_flags=flags)
     # bit 0: a stream outgrew its 256 bytes and was cut (possible only when a table covers many
     # more tokens than a stream holds); reported, and then the round trip is not checked
     status = int(enc.status.item())
@@ -182,7 +190,7 @@ def run_workload(name, steps, warmup, fmt="vllm", copy_probe=False, keep=False, 
     out = torch.empty_like(kv)
 
     def encode():
-        codec.encode_kv(kv, kb, vb, chunk_tokens=chunk, max_bins=max_bins, workspace=workspace, out=enc, fmt=fmt)
+        codec.encode_kv(kv, kb, vb, chunk_tokens=chunk, max_bins=max_bins, workspace=workspace, out=enc, fmt=fmt, _test_flags=flags)
 
     def decode():
         codec.decode_encoded(enc, kb, vb, fmt=fmt, out=out)
@@ -403,6 +411,8 @@ def main():
     ap.add_argument("--cpu-sample-tokens", type=int, default=8192)
     ap.add_argument("--fmt", default="vllm", choices=["vllm", "huggingface"],
                     help="layout of the KV tensor: [L,2,T,H,D] (vllm, the metric's layout) or [L,2,H,T,D]")
+    ap.add_argument("--encode-form", default="default", choices=sorted(ENCODE_FORMS),
+                    help="force one of the library's internal forms of the encode call (same bytes; for profiles)")
     ap.add_argument("--no-issue-probe", action="store_true",
                     help="skip the engine-clock sampler and the instruction-issue calibration (valu_issue)")
     ap.add_argument("--copy-probe", action="store_true",
@@ -421,7 +431,7 @@ def main():
     torch.cuda.set_device(0)
     fmt = args.fmt
     r = run_workload(args.workload, args.steps, args.warmup, fmt=fmt, copy_probe=args.copy_probe, keep=True,
-                     ramp_ms=args.clock_ramp_ms, sample_clock=not args.no_issue_probe)
+                     ramp_ms=args.clock_ramp_ms, sample_clock=not args.no_issue_probe, encode_form=args.encode_form)
     kept = r.pop("_keep")
     ab = r["algorithmic_bytes"]
     kv_bytes = r["kv_bytes"]
@@ -448,6 +458,7 @@ def main():
             "value_is": "fp16 KV bytes encoded plus decoded per second of a full encode+decode step",
             "kv_bytes": kv_bytes,
             "streams": r["streams"],
+            **({"encode_form": args.encode_form} if args.encode_form != "default" else {}),
         },
         "encode_GBps": round(r["encode_GBps"], 3),
         "decode_GBps": round(r["decode_GBps"], 3),
